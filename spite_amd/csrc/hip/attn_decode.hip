@@ -31,7 +31,7 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                         const int* __restrict__ block_table, int max_blocks, int H, int G, int ps, int vis,
                         int span, float scale_log2e, float cap_ratio, int n_splits,
-                        const float* __restrict__ slopes, float inv_scale, int Gv) {
+                        const float* __restrict__ slopes, float inv_scale, int Gv, const float* __restrict__ sinks) {
     constexpr int NC = HD / 32;      // 32-wide chunks of the head for the score product
     constexpr int ND = HD / 16;      // 16-row tiles of the output
     constexpr int ROW = HD + 2;      // partial record: output, max, sum
@@ -59,6 +59,9 @@ void attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_p
         qf[c] = n < QH ? *(const bf16x8*)(q + ((size_t)t * H + g * QH + n) * HD + c * 32 + qd * 8) : zero8;
 
     float m_run = -INFINITY, l_run = 0.f;
+    // a sink (one more term exp(sinks[head]) in the softmax's denominator, with no key and no value) is the
+    // first term of the first split's first wave: it sets the running maximum, in the exponent's units, and counts once
+    if (sinks && split == 0 && wave == 0 && n < QH) { m_run = sinks[g * QH + n] * 1.4426950408889634f; l_run = 1.f; }
     f32x4 o[ND];
 #pragma unroll
     for (int d = 0; d < ND; ++d) o[d] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -243,7 +246,7 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
                                  const int* positions, const int* seq_of_token, const int* block_table,
                                  int max_blocks, int T, int H, int G, int hd, int page_size, int vis, int span,
                                  float scale, float softcap, const float* slopes, int n_splits, int value_heads,
-                                 hipStream_t st) {
+                                 const float* sinks, hipStream_t st) {
     SP_REQUIRE(softcap >= 0.f && scale > 0.f, "attn_decode: scale %g, score cap %g", scale, softcap);
     // value pages [pages][value_heads][hd][page]: kv head g reads value head g % value_heads (0: as many as kv heads)
     if (value_heads <= 0) value_heads = G;
@@ -261,13 +264,13 @@ extern "C" int spite_attn_decode(const void* q, const void* k_pages, const void*
     const size_t sh = (size_t)4 * 16 * (hd + 2) * sizeof(float);
     if (hd == 128) {
         attn_decode_kernel<128><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale, value_heads);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale, value_heads, sinks);
         SP_LAUNCH_CHECK("attn_decode");
         if (n_splits > 1)
             attn_decode_combine_kernel<128><<<dim3(T, H), 128, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
     } else {
         attn_decode_kernel<64><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale, value_heads);
+            (float*)workspace, (bf16*)out, positions, seq_of_token, block_table, max_blocks, H, G, page_size, vis, span, sl, cr, n_splits, slopes, 1.0f / scale, value_heads, sinks);
         SP_LAUNCH_CHECK("attn_decode");
         if (n_splits > 1)
             attn_decode_combine_kernel<64><<<dim3(T, H), 64, 0, st>>>((const float*)workspace, (bf16*)out, H, n_splits);
@@ -313,5 +316,5 @@ extern "C" int spite_attn_decode_static(const void* q, const void* k_pages, cons
     SP_REQUIRE(e == hipSuccess && ptr != nullptr, "attn_decode_static: no address for the scratch array: %s",
                hipGetErrorString(e));
     return spite_attn_decode(q, k_pages, v_pages, out, ptr, positions, seq_of_token, block_table, max_blocks, T, H, G,
-                             hd, page_size, vis, span, scale, 0.f, nullptr, n_splits, 0, st);
+                             hd, page_size, vis, span, scale, 0.f, nullptr, n_splits, 0, nullptr, st);
 }

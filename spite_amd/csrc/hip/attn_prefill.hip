@@ -56,7 +56,8 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
                          const int* __restrict__ positions, const int* __restrict__ cu_seqlens, int n_seqs,
                          const int* __restrict__ block_table, int max_blocks, int tile_q,
                          int H, int G, int ps, int vis, int span, float scale_log2e, float cap_ratio,
-                         const float* __restrict__ slopes, float inv_scale, int n_splits, int Gv) {
+                         const float* __restrict__ slopes, float inv_scale, int n_splits, int Gv,
+                         const float* __restrict__ sinks) {
     constexpr int NS = HD / 16;                      // steps of 16 head elements in the score product
     constexpr int NDT = HD / 32;                     // 32-row tiles of the output
     constexpr int NC = HD / 32;                      // chunks of a K tile row
@@ -118,6 +119,9 @@ void attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_
     // m_run: the running maximum of the scaled scores (in the exponent's units); l_run: this
     // lane's part of the running sum (the two lanes of a column meet at the end)
     float m_run = -INFINITY, l_run = 0.f;
+    // a sink (one more term exp(sinks[head]) in the softmax's denominator, with no key and no value) is the
+    // first term of the first split's sum: it sets the running maximum, in the exponent's units, and counts once
+    if (sinks && live && split == 0) { m_run = sinks[head] * 1.4426950408889634f; l_run = hh == 0 ? 1.f : 0.f; }
     f32x16 o[NDT];
 #pragma unroll
     for (int d = 0; d < NDT; ++d)
@@ -423,7 +427,7 @@ template <int HD, bool EXTRA>
 static int launch_prefill(const void* q, const void* k_pages, const void* v_pages, void* out, float* part, const int* positions,
                           const int* cu_seqlens, int n_seqs, const int* block_table, int max_blocks, int tile_q,
                           long n_tiles, int H, int G, int page_size, int vis, int span, float sl, float cr,
-                          const float* slopes, float inv_scale, int n_splits, int Gv, hipStream_t st) {
+                          const float* slopes, float inv_scale, int n_splits, int Gv, const float* sinks, hipStream_t st) {
     const size_t sh = (size_t)2 * 2 * PF_KEYS * HD * sizeof(bf16);
     static bool allowed = false;          // one flag per instantiation: more LDS than the default limit
     if (!allowed) {
@@ -433,7 +437,7 @@ static int launch_prefill(const void* q, const void* k_pages, const void* v_page
     }
     attn_prefill_kernel<HD, EXTRA><<<dim3((unsigned)(n_tiles * G * n_splits)), 512, sh, st>>>((const bf16*)q, (const bf16*)k_pages,
         (const bf16*)v_pages, (bf16*)out, part, positions, cu_seqlens, n_seqs, block_table, max_blocks, tile_q, H, G, page_size,
-        vis, span, sl, cr, slopes, inv_scale, n_splits, Gv);
+        vis, span, sl, cr, slopes, inv_scale, n_splits, Gv, sinks);
     SP_LAUNCH_CHECK("attn_prefill");
     return 0;
 }
@@ -469,12 +473,13 @@ extern "C" int spite_attn_prefill_splits(const int* counts, int n_seqs, int H, i
 // tile's keys are dealt to that many workgroups, whose partial results go to `workspace`
 // (spite_attn_prefill_workspace bytes) and are joined by a second kernel.  `slopes` (device,
 // fp32 [H], or null): a bias slopes[head] * (key position - query position) added to the scaled
-// scores before the cap.
+// scores before the cap.  `sinks` (device, fp32 [H], or null): one more term exp(sinks[head]) in the
+// denominator of every softmax of that head.
 extern "C" int spite_attn_prefill(const void* q, const void* k_pages, const void* v_pages, void* out, void* workspace,
                                   const int* positions, const int* cu_seqlens, const int* counts, int n_seqs,
                                   const int* block_table, int max_blocks, int H, int G, int hd, int page_size,
                                   int vis, int span, float scale, float softcap, const float* slopes, int n_splits,
-                                  int value_heads, hipStream_t st) {
+                                  int value_heads, const float* sinks, hipStream_t st) {
     SP_REQUIRE(softcap >= 0.f && scale > 0.f, "attn_prefill: scale %g, score cap %g", scale, softcap);
     // value pages [pages][value_heads][hd][page]: kv head g reads value head g % value_heads (0: as many as kv heads)
     if (value_heads <= 0) value_heads = G;
@@ -498,7 +503,7 @@ extern "C" int spite_attn_prefill(const void* q, const void* k_pages, const void
     const float sl = scale * 1.4426950408889634f, cr = softcap > 0.f ? scale / softcap : 0.f;
     const bool extra = cr > 0.f || slopes != nullptr;
 #define SP_PF(HDV, EX) launch_prefill<HDV, EX>(q, k_pages, v_pages, out, (float*)workspace, positions, cu_seqlens, n_seqs, \
-        block_table, max_blocks, tile_q, tiles, H, G, page_size, vis, span, sl, cr, slopes, 1.0f / scale, n_splits, value_heads, st)
+        block_table, max_blocks, tile_q, tiles, H, G, page_size, vis, span, sl, cr, slopes, 1.0f / scale, n_splits, value_heads, sinks, st)
     const int rc = hd == 128 ? (extra ? SP_PF(128, true) : SP_PF(128, false)) : (extra ? SP_PF(64, true) : SP_PF(64, false));
 #undef SP_PF
     if (rc != 0 || n_splits == 1) return rc;

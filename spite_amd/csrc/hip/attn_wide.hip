@@ -21,7 +21,9 @@
 // whole q or k part again).  The row holds [HQ*D | GK*D | GV*Vd | ...] (`ld` elements to the next
 // row).  x = row + bias; with `wq` / `wk` the q and the k region are each divided by the root mean
 // square of the whole region and multiplied by their weights; then the first `rot` elements
-// of every q and k head turn by pos * inv_freq[i] in pairs (i, i + rot/2); with `inv_freq_v` the
+// of every q and k head turn by pos * inv_freq[i] in pairs (i, i + rot/2), sine and cosine both
+// times `rot_mag` (1: a pure rotation; frequency scalings that stretch the context bring a
+// constant above 1 that sharpens the scores of the turning part); with `inv_freq_v` the
 // values turn by pos * inv_freq_v[m] in pairs (m, m + Vd/2).  Keys go to [page][GK][offset][Dp],
 // values to [page][GV][Vd][offset] (or the operand order of common.h).  Dp >= D is the width that
 // queries and keys are stored with: the elements behind D are written as zeros (a head narrower than
@@ -32,7 +34,7 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
                         const float* __restrict__ wq, const float* __restrict__ wk, float eps,
                         T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
                         const int* __restrict__ positions, const int* __restrict__ slot_map,
-                        const float* __restrict__ inv_freq, int rot, const float* __restrict__ inv_freq_v,
+                        const float* __restrict__ inv_freq, int rot, float rot_mag, const float* __restrict__ inv_freq_v,
                         int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp, int hpb) {
     extern __shared__ float sm[];
     __shared__ float red[WIDE_NT / 64];
@@ -45,7 +47,7 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
     const float pos = (float)positions[t];
     const T* row = qkv + (size_t)t * ld;
     const int Nq = HQ * D, Nk = GK * D;
-    for (int i = tid; i < rh; i += WIDE_NT) sincosf(pos * inv_freq[i], &sn[i], &cs[i]);
+    for (int i = tid; i < rh; i += WIDE_NT) { float sv, cv; sincosf(pos * inv_freq[i], &sv, &cv); sn[i] = sv * rot_mag; cs[i] = cv * rot_mag; }
     for (int i = tid; i < vh; i += WIDE_NT) sincosf(pos * inv_freq_v[i], &snv[i], &csv[i]);
     const int slot = slot_map ? slot_map[t] : -1;
     // this workgroup's heads [h_lo, h_hi) of the HQ + GK + GV; keys and values only where the token has a cache row
@@ -131,7 +133,7 @@ void qkv_prepare_vec_kernel(const bf16* __restrict__ qkv, int ld, const float* _
                             const float* __restrict__ wq, const float* __restrict__ wk, float eps,
                             bf16* __restrict__ q_out, bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
                             const int* __restrict__ positions, const int* __restrict__ slot_map,
-                            const float* __restrict__ inv_freq, int rot, const float* __restrict__ inv_freq_v,
+                            const float* __restrict__ inv_freq, int rot, float rot_mag, const float* __restrict__ inv_freq_v,
                             int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp, int hpb) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
     __shared__ float red[WIDE_NT / 64];
@@ -144,7 +146,7 @@ void qkv_prepare_vec_kernel(const bf16* __restrict__ qkv, int ld, const float* _
     const float pos = (float)positions[t];
     const bf16* row = qkv + (size_t)t * ld;
     const int Nq = HQ * D, Nk = GK * D;
-    for (int i = tid; i < rh; i += WIDE_NT) sincosf(pos * inv_freq[i], &sn[i], &cs[i]);
+    for (int i = tid; i < rh; i += WIDE_NT) { float sv, cv; sincosf(pos * inv_freq[i], &sv, &cv); sn[i] = sv * rot_mag; cs[i] = cv * rot_mag; }
     for (int i = tid; i < vh; i += WIDE_NT) sincosf(pos * inv_freq_v[i], &snv[i], &csv[i]);
     const int slot = slot_map ? slot_map[t] : -1;
     const int h_lo = blockIdx.y * hpb, h_end = h_lo + hpb;
@@ -222,7 +224,7 @@ void qkv_prepare_vec_kernel(const bf16* __restrict__ qkv, int ld, const float* _
 
 extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float* bias, const float* wq, const float* wk,
                                  float eps, void* q_out, void* k_pages, void* v_pages, const int* positions,
-                                 const int* slot_map, const float* inv_freq, int rot, const float* inv_freq_v,
+                                 const int* slot_map, const float* inv_freq, int rot, float rot_mag, const float* inv_freq_v,
                                  int T, int HQ, int GK, int GV, int D, int Vd, int page_size, int k_tiled, int v_tiled,
                                  int Dp, hipStream_t st) {
     if (Dp <= 0) Dp = D;
@@ -251,16 +253,16 @@ extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float
         && al(bias, 16) && al(wq, 16) && al(wk, 16)) {
         // (the sine and cosine tables are read four at a time: the second starts rot/2 floats behind the first)
         qkv_prepare_vec_kernel<<<grid, WIDE_NT, sh, st>>>((const bf16*)qkv, ld, bias, wq, wk, eps, (bf16*)q_out, (bf16*)k_pages,
-            (bf16*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
+            (bf16*)v_pages, positions, slot_map, inv_freq, rot, rot_mag, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
         SP_LAUNCH_CHECK("qkv_prepare");
         return 0;
     }
     if (dtype == SP_F32)
         qkv_prepare_kernel<float><<<grid, WIDE_NT, sh, st>>>((const float*)qkv, ld, bias, wq, wk, eps, (float*)q_out, (float*)k_pages,
-            (float*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
+            (float*)v_pages, positions, slot_map, inv_freq, rot, rot_mag, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
     else if (dtype == SP_BF16)
         qkv_prepare_kernel<bf16><<<grid, WIDE_NT, sh, st>>>((const bf16*)qkv, ld, bias, wq, wk, eps, (bf16*)q_out, (bf16*)k_pages,
-            (bf16*)v_pages, positions, slot_map, inv_freq, rot, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
+            (bf16*)v_pages, positions, slot_map, inv_freq, rot, rot_mag, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
     else return sp_fail("qkv_prepare: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("qkv_prepare");
     return 0;
@@ -269,7 +271,9 @@ extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float
 // ------------------------------------------------------------------ the plain attention kernel
 // One wave per (token, query head).  Keys are walked in tiles of 64 that start at the first
 // visible key, so the order of every sum depends on the query's position alone: a token gives
-// the same bits whether it comes in a whole prompt, a portion or alone.
+// the same bits whether it comes in a whole prompt, a portion or alone.  With `sinks` (fp32 [HQ])
+// every head's softmax has one more term in its denominator, exp(sinks[h]): a score that is not
+// scaled, belongs to no key and brings no value.
 #define WIDE_MAX_V 8   // value widths up to 512
 
 template <typename T, typename TO>
@@ -278,7 +282,7 @@ void attn_wide_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
                       TO* __restrict__ out, const int* __restrict__ positions,
                       const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                       int max_blocks, int HQ, int GK, int GV, int D, int Vd, int ps, int vis, int span, float scale,
-                      int k_tiled, int v_tiled) {
+                      int k_tiled, int v_tiled, const float* __restrict__ sinks) {
     extern __shared__ float smem[];
     float* q_sh = smem;                 // [D]
     float* p_sh = smem + D;             // [64]
@@ -293,7 +297,8 @@ void attn_wide_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
     for (int c = lane; c < D; c += 64) q_sh[c] = to_f32<T>(qr[c]);
     __syncthreads();
 
-    float m = -INFINITY, l = 0.f;
+    // the sink is the softmax's first term: it sets the running maximum and counts once
+    float m = sinks ? sinks[h] : -INFINITY, l = sinks ? 1.f : 0.f;
     float o[WIDE_MAX_V];
 #pragma unroll
     for (int u = 0; u < WIDE_MAX_V; ++u) o[u] = 0.f;
@@ -350,7 +355,7 @@ void attn_wide_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
 extern "C" int spite_attn_wide(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype, int out_dtype,
                                const int* positions, const int* seq_of_token, const int* block_table,
                                int max_blocks, int T, int HQ, int GK, int GV, int D, int Vd, int page_size, int vis, int span,
-                               float scale, int k_tiled, int v_tiled, hipStream_t st) {
+                               float scale, int k_tiled, int v_tiled, const float* sinks, hipStream_t st) {
     SP_REQUIRE(T >= 0 && HQ > 0 && GK > 0 && GV > 0 && HQ % GK == 0 && GK % GV == 0,
                "attention: %d query heads over %d key heads over %d value heads", HQ, GK, GV);
     SP_REQUIRE(D > 0 && D <= 4096 && Vd > 0 && Vd <= 64 * WIDE_MAX_V, "attention: keys of %d, values of %d (at most %d)", D, Vd, 64 * WIDE_MAX_V);
@@ -363,7 +368,7 @@ extern "C" int spite_attn_wide(const void* q, const void* k_pages, const void* v
     dim3 grid(T, HQ);
     const size_t sh = (size_t)(D + 64) * sizeof(float) + 128 * sizeof(int);
 #define SP_AW(TI, TO) attn_wide_kernel<TI, TO><<<grid, 64, sh, st>>>((const TI*)q, (const TI*)k_pages, (const TI*)v_pages, (TO*)out, \
-        positions, seq_of_token, block_table, max_blocks, HQ, GK, GV, D, Vd, page_size, vis, span, scale, k_tiled, v_tiled)
+        positions, seq_of_token, block_table, max_blocks, HQ, GK, GV, D, Vd, page_size, vis, span, scale, k_tiled, v_tiled, sinks)
     if (dtype == SP_F32 && out_dtype == SP_F32) SP_AW(float, float);
     else if (dtype == SP_BF16 && out_dtype == SP_BF16) SP_AW(bf16, bf16);
     else if (dtype == SP_BF16 && out_dtype == SP_F32) SP_AW(bf16, float);

@@ -127,11 +127,12 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return t;
 }
 
-// The gate's activation in a gated product act(gate) * up: SP_ACT_SILU g * sigmoid(g), or
-// SP_ACT_GELU_TANH 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))).  `fast`: the short exponential
-// (the bfloat16 products); the 32-bit path takes the accurate routines.
-enum { SP_ACT_NONE = 0, SP_ACT_SILU = 1, SP_ACT_GELU_TANH = 2 };
+// The gate's activation in a gated product act(gate) * up: SP_ACT_SILU g * sigmoid(g),
+// SP_ACT_GELU_TANH 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))), or SP_ACT_RELU max(g, 0).
+// `fast`: the short exponential (the bfloat16 products); the 32-bit path takes the accurate routines.
+enum { SP_ACT_NONE = 0, SP_ACT_SILU = 1, SP_ACT_GELU_TANH = 2, SP_ACT_RELU = 3 };
 __device__ __forceinline__ float sp_gate_act(float g, int act, bool fast) {
+    if (act == SP_ACT_RELU) return fmaxf(g, 0.f);
     if (act == SP_ACT_GELU_TANH) {
         const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
         // tanh(z) = 1 - 2 / (exp(2z) + 1): no cancellation where it matters, exact limits at both ends

@@ -1,9 +1,12 @@
 // Routers that pick several experts a token, and what surrounds their grouped products.
 //
-// router_topk: scores s = sigmoid(z) of the router's fp32 logits z [T, E]; the `top` experts with
-// the largest choice scores s + bias (bias may be null; the lowest index wins among equals) are
-// taken, and an expert's weight is its score s without the bias, divided by the sum of the taken
-// scores if `renorm`.  Outputs expert[t*top + j] and weight[t*top + j] in the order of choice:
+// router_topk: from the router's fp32 logits z [T, E] the `top` experts with the largest choice
+// values are taken (the lowest index wins among equals), and each gets a weight.  Two ways of scoring:
+//   sigmoid (mode 0): scores s = sigmoid(z); the choice goes by s + bias (bias may be null); an expert's
+//     weight is its score s without the bias, divided by the sum of the taken scores if `renorm`;
+//   softmax over the taken (mode 1): the choice goes by z + bias; the weights are the softmax of the taken
+//     experts' logits z alone (they add up to one; `renorm` has nothing left to do).
+// Outputs expert[t*top + j] and weight[t*top + j] in the order of choice:
 // "virtual tokens" t*top + j that the expert plan (moe_plan with its fan) sorts by expert.
 // moe_combine: out[t] = sum_j weight[t*top + j] * y[t*top + j] (+ extra[t]) in fp32, j in order.
 // gated_rows: g[t] = gelu_tanh(a[t]) * table[ids[t]][col0 .. col0 + n): a gate on a per-token row
@@ -14,7 +17,7 @@
 
 __global__ __launch_bounds__(256)
 void router_topk_kernel(const float* __restrict__ logits, const float* __restrict__ bias, int* __restrict__ expert,
-                        float* __restrict__ weight, int T, int E, int top, int renorm) {
+                        float* __restrict__ weight, int T, int E, int top, int renorm, int mode) {
     const int lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (t >= T) return;
@@ -24,12 +27,13 @@ void router_topk_kernel(const float* __restrict__ logits, const float* __restric
         const int e = lane + u * 64;
         s[u] = 0.f; c[u] = -INFINITY;
         if (e < E) {
-            s[u] = 1.0f / (1.0f + expf(-logits[(size_t)t * E + e]));
+            const float z = logits[(size_t)t * E + e];
+            s[u] = mode == 1 ? z : 1.0f / (1.0f + expf(-z));
             c[u] = s[u] + (bias ? bias[e] : 0.f);
             if (!(c[u] == c[u])) c[u] = -INFINITY;          // a NaN is never chosen before a number
         }
     }
-    float sum = 0.f;
+    float sum = 0.f, top_z = -INFINITY;          // mode 1: the sum of exp(z - top_z) over the taken so far
     float mine_w = 0.f; int mine_e = 0;
     for (int j = 0; j < top; ++j) {
         float best = -INFINITY; int be = 0x7fffffff; float bs = 0.f;
@@ -46,9 +50,21 @@ void router_topk_kernel(const float* __restrict__ logits, const float* __restric
         // a taken expert leaves the contest: its mark lies below every score
 #pragma unroll
         for (int u = 0; u < TOPK_MAX_PER_LANE; ++u) if (lane + u * 64 == be) c[u] = -INFINITY;
-        sum += bs;
+        if (mode == 1) {
+            const float nz = fmaxf(top_z, bs);
+            sum = sum * expf(top_z - nz) + expf(bs - nz);        // (exp(-inf) = 0 at the first)
+            top_z = nz;
+        } else {
+            sum += bs;
+        }
         if (lane == j % 64 && j < 64) { mine_w = bs; mine_e = be; }
         if (j >= 64 && lane == 0) { expert[(size_t)t * top + j] = be; weight[(size_t)t * top + j] = bs; }
+    }
+    if (mode == 1) {
+        const float inv = 1.0f / sum;
+        if (lane < top && lane < 64) { expert[(size_t)t * top + lane] = mine_e; weight[(size_t)t * top + lane] = expf(mine_w - top_z) * inv; }
+        if (top > 64 && lane == 0) for (int j = 64; j < top; ++j) weight[(size_t)t * top + j] = expf(weight[(size_t)t * top + j] - top_z) * inv;
+        return;
     }
     const float inv = renorm ? 1.0f / fmaxf(sum, 1e-20f) : 1.0f;
     if (lane < top && lane < 64) { expert[(size_t)t * top + lane] = mine_e; weight[(size_t)t * top + lane] = mine_w * inv; }
@@ -56,11 +72,12 @@ void router_topk_kernel(const float* __restrict__ logits, const float* __restric
 }
 
 extern "C" int spite_router_topk(const float* logits, const float* bias, int* expert, float* weight, int T, int E, int top,
-                                 int renorm, hipStream_t st) {
+                                 int renorm, int mode, hipStream_t st) {
+    SP_REQUIRE(mode == 0 || mode == 1, "router_topk: scoring %d", mode);
     SP_REQUIRE(T >= 0 && E > 0 && E <= 64 * TOPK_MAX_PER_LANE, "router_topk: %d experts, at most %d", E, 64 * TOPK_MAX_PER_LANE);
     SP_REQUIRE(top > 0 && top <= E, "router_topk: %d of %d experts", top, E);
     if (T == 0) return 0;
-    router_topk_kernel<<<(T + 3) / 4, 256, 0, st>>>(logits, bias, expert, weight, T, E, top, renorm);
+    router_topk_kernel<<<(T + 3) / 4, 256, 0, st>>>(logits, bias, expert, weight, T, E, top, renorm, mode);
     SP_LAUNCH_CHECK("router_topk");
     return 0;
 }

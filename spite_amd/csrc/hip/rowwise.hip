@@ -1,4 +1,5 @@
-// Small row-wise kernels: the token shift of a mixer's input and an activation applied in place.
+// Small row-wise kernels: the token shift of a mixer's input, an activation applied in place and a
+// constant on fp32 rows (the logits of a model whose output has one).
 #include "common.h"
 
 // ------------------------------------------------------------------ token shift
@@ -99,5 +100,20 @@ extern "C" int spite_act_rows(void* x, int dtype, size_t n, int act, hipStream_t
         else return sp_fail("act_rows: unknown dtype %d", dtype);
     }
     SP_LAUNCH_CHECK("act_rows");
+    return 0;
+}
+
+// ------------------------------------------------------------------ a constant on fp32 rows, in place
+__global__ __launch_bounds__(256)
+void scale_rows_kernel(float* __restrict__ x, size_t n, float c) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) x[i] *= c;
+}
+
+extern "C" int spite_scale_rows(float* x, size_t n, float c, hipStream_t st) {
+    if (n == 0) return 0;
+    const int blocks = (int)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+    scale_rows_kernel<<<blocks, 256, 0, st>>>(x, n, c);
+    SP_LAUNCH_CHECK("scale_rows");
     return 0;
 }

@@ -18,7 +18,7 @@ from . import build
 F32, BF16 = 0, 1
 VIS = build.visibility_codes()      # "full", "chunk", "window": name -> code
 # the gate's activation of a gated product act(gate) * up, as the kernels number them (True: silu)
-GATE_ACTS = {False: 0, None: 0, True: 1, "silu": 1, "gelu_tanh": 2}
+GATE_ACTS = {False: 0, None: 0, True: 1, "silu": 1, "gelu_tanh": 2, "relu": 3}
 # an activation of a plain product's own (no gate), as the kernels number them; the bf16 weight-stream and
 # tiled products take it in their epilogue, in the bits above the gate's code
 UNARY_ACTS = {"gelu": 1, "gelu_tanh": 2, "silu": 3}
@@ -51,11 +51,11 @@ def lib():
             "spite_sample_rows": [P, I, I, I, P, P, P, P],
             "spite_filter_rows": [P, I, I, I, P, P, P, P],
             "spite_gemm_skinny": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, I, I, I, P],
-            "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, I, P],
+            "spite_attn_decode": [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, F, P, I, I, P, P],
             "spite_gemm_mfma": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled": [P, I, P, L, P, I, I, I, I, I, P, I, P, P, P, I, I, P],
             "spite_gemm_tiled_split": [P, I, P, P, I, I, I, I, I, I, P, P],
-            "spite_attn_prefill": [P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, F, P, I, I, P],
+            "spite_attn_prefill": [P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, F, P, I, I, P, P],
             "spite_attn_prefill_splits": [P, I, I, I, L],
             "spite_argmax_rows": [P, I, I, I, P, P, P, P],
             "spite_stream_read": [P, c_size_t, P, I, P],
@@ -63,14 +63,18 @@ def lib():
             "spite_latent_prepare": [P, I, P, I, P, P, I, P, P, P, P, F, I, I, I, I, I, I, I, P, P, P],
             "spite_attn_latent_generic": [P, P, P, I, P, P, P, I, I, I, I, I, I, I, I, F, P],
             "spite_attn_latent_mfma": [P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, F, P, I, I, P],
-            "spite_router_topk": [P, P, P, P, I, I, I, I, P],
+            "spite_router_topk": [P, P, P, P, I, I, I, I, I, P],
             "spite_moe_combine": [P, P, P, P, I, I, I, P],
             "spite_gated_rows": [P, I, P, P, I, I, I, P, I, I, P],
-            "spite_qkv_prepare": [P, I, I, P, P, P, F, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, I, I, I, P],
-            "spite_attn_wide": [P, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, I, F, I, I, P],
+            "spite_qkv_prepare": [P, I, I, P, P, P, F, P, P, P, P, P, P, I, F, P, I, I, I, I, I, I, I, I, I, I, P],
+            "spite_attn_wide": [P, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, I, F, I, I, P, P],
             "spite_attn_finish": [P, I, P, I, P, P, P, I, I, I, I, I, F, F, F, P],
             "spite_token_shift": [P, P, I, P, P, P, P, P, I, I, I, P],
             "spite_act_rows": [P, I, c_size_t, I, P],
+            "spite_scale_rows": [P, c_size_t, F, P],
+            "spite_channel_decay": [P, P, I, I, F, P],
+            "spite_linear_attn_scan": [P, P, P, I, I, I, I, P, P, F, P, I, P, P, I, P, I, I, I, I, P],
+            "spite_gated_group_norm": [P, P, I, P, I, P, I, I, I, I, F, I, P],
         }
         for name, args in sigs.items():
             fn = getattr(l, name)
@@ -444,11 +448,12 @@ def attn_decode_workspace(T, H, hd, n_splits) -> int:
 
 
 def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, block_table, T, H, G, hd,
-                page_size, vis, span, scale, n_splits, softcap=0.0, slopes=None, value_heads=None):
+                page_size, vis, span, scale, n_splits, softcap=0.0, slopes=None, value_heads=None, sinks=None):
     """Split-KV decode attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32
     keys, in operand order): every row of q is one query against its request's cache.
     ``value_heads``: the value pages hold fewer heads than the key pages (kv head g reads value
-    head g % value_heads)."""
+    head g % value_heads).  ``sinks`` (fp32 [H] or None): one more term exp(sinks[h]) in every
+    softmax's denominator."""
     if q.dtype != torch.bfloat16:
         raise KernelError(f"attn_decode: bfloat16 only, got {q.dtype}")
     if q.numel() < T * H * hd or out.numel() < T * H * hd:
@@ -464,7 +469,7 @@ def attn_decode(q, k_pages, v_pages, out, workspace, positions, seq_of_token, bl
         _ptr(workspace, "workspace"), _ptr(positions, "positions", torch.int32),
         _ptr(seq_of_token, "seq_of_token", torch.int32), _ptr(block_table, "block_table", torch.int32),
         block_table.shape[1], T, H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), float(softcap),
-        _slopes(slopes, H), int(n_splits), int(value_heads or 0), _stream()), "attn_decode")
+        _slopes(slopes, H), int(n_splits), int(value_heads or 0), _slopes(sinks, H), _stream()), "attn_decode")
 
 
 def gemm_mfma(a, w, y, M, N, K, *, offsets=None, n_groups=1, a_rows=None, a_scale=None, y_rows=None, glu=False,
@@ -557,7 +562,8 @@ def attn_prefill_workspace(counts, H, G, hd, n_splits) -> int:
 
 
 def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_table,
-                 H, G, hd, page_size, vis, span, scale, n_splits=1, scratch=None, softcap=0.0, slopes=None, value_heads=None):
+                 H, G, hd, page_size, vis, span, scale, n_splits=1, scratch=None, softcap=0.0, slopes=None, value_heads=None,
+                 sinks=None):
     """Prefill attention on MFMA (bf16; head sizes 64 and 128; pages of a multiple of 32 keys, in
     operand order).
     ``counts``: the number of query tokens of every request of the step, on the host, in the
@@ -565,7 +571,8 @@ def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_
     ``n_splits`` > 1 deals every tile's keys to that many workgroups; ``scratch`` (fp32,
     ``attn_prefill_workspace`` bytes) then holds their partial results.
     ``slopes`` (fp32 [H] or None): a bias slopes[head] * (key position - query position) on the
-    scaled scores, before the cap."""
+    scaled scores, before the cap.  ``sinks`` (fp32 [H] or None): one more term exp(sinks[h]) in
+    every softmax's denominator."""
     if q.dtype != torch.bfloat16:
         raise KernelError(f"attn_prefill: bfloat16 only, got {q.dtype}")
     counts = np.ascontiguousarray(counts, dtype=np.int32)
@@ -588,7 +595,7 @@ def attn_prefill(q, k_pages, v_pages, out, positions, cu_seqlens, counts, block_
         _ptr(positions, "positions", torch.int32), _ptr(cu_seqlens, "cu_seqlens", torch.int32),
         counts.ctypes.data, n_seqs, _ptr(block_table, "block_table", torch.int32), block_table.shape[1],
         H, G, hd, page_size, VIS[vis], int(span or 0), float(scale), float(softcap), _slopes(slopes, H), n_splits,
-        int(value_heads or 0), _stream()), "attn_prefill")
+        int(value_heads or 0), _slopes(sinks, H), _stream()), "attn_prefill")
 
 
 def _slopes(slopes, H):
@@ -681,16 +688,23 @@ def attn_latent_generic(q, kv_pages, out, positions, seq_of_token, block_table, 
 
 
 # -------------------------------------------------------------------------------------------- several experts a token
-def router_topk(logits, bias, expert, weight, top, renorm=False):
+ROUTER_SCORING = {"sigmoid": 0, "softmax_taken": 1}
+
+
+def router_topk(logits, bias, expert, weight, top, renorm=False, scoring="sigmoid"):
     """From fp32 router logits [T, E]: scores sigmoid(z); the ``top`` experts with the largest
     score + bias (bias fp32 [E] or None; lowest index among equals) into expert[T*top], their
-    scores (without the bias; divided by their sum with ``renorm``) into weight[T*top]."""
+    scores (without the bias; divided by their sum with ``renorm``) into weight[T*top].  With
+    ``scoring`` = ``softmax_taken`` the choice goes by z + bias and the weights are the softmax over the
+    taken experts' logits."""
     T, E = logits.shape
+    if scoring not in ROUTER_SCORING:
+        raise KernelError(f"router_topk: scoring {scoring!r} (known: {sorted(ROUTER_SCORING)})")
     if expert.numel() < T * top or weight.numel() < T * top or (bias is not None and bias.numel() != E):
         raise KernelError("router_topk: outputs too small or bias of the wrong size")
     _check(lib().spite_router_topk(_ptr(logits, "logits", torch.float32), _ptr(bias, "bias", torch.float32, True),
                                    _ptr(expert, "expert", torch.int32), _ptr(weight, "weight", torch.float32),
-                                   T, E, int(top), int(bool(renorm)), _stream()), "router_topk")
+                                   T, E, int(top), int(bool(renorm)), ROUTER_SCORING[scoring], _stream()), "router_topk")
 
 
 def moe_combine(y, weight, extra, out, T, top):
@@ -772,12 +786,13 @@ def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg,
 # -------------------------------------------------------------------------------------------- keys and values of unequal shape
 def qkv_prepare(qkv, q_out, k_pages, v_pages, positions, slot_map, HQ, GK, GV, D, Vd, page_size, *, bias=None,
                 norm_q=None, norm_k=None, eps=0.0, inv_freq=None, rot=0, inv_freq_v=None, write_kv=True,
-                k_tiled=False, v_tiled=False, stored_dim=None):
+                k_tiled=False, v_tiled=False, stored_dim=None, rot_magnitude=1.0):
     """Between a fused projection and the cache (see attn_wide.hip).  qkv: rows that begin with
     [HQ*D | GK*D | GV*Vd] (further columns are left alone); ``bias`` fp32 over those; ``norm_q`` /
     ``norm_k`` (fp32 [HQ*D], [GK*D]): weights of an RMS norm over the whole q and the whole k part;
     ``inv_freq`` (fp32 [rot/2]): the first ``rot`` elements of every q and k head turn in pairs
-    (i, i + rot/2); ``inv_freq_v`` (fp32 [Vd/2]): the values turn in pairs (m, m + Vd/2).  q_out
+    (i, i + rot/2), sine and cosine times ``rot_magnitude``; ``inv_freq_v`` (fp32 [Vd/2]): the values turn in
+    pairs (m, m + Vd/2).  q_out
     [T, HQ*Dp]; key pages [pages, GK, page_size, Dp]; value pages [pages, GV, Vd, page_size], with
     Dp = ``stored_dim`` (default D): queries and keys are stored that wide, zeros behind their D."""
     T = qkv.shape[0]
@@ -806,15 +821,19 @@ def qkv_prepare(qkv, q_out, k_pages, v_pages, positions, slot_map, HQ, GK, GV, D
         _ptr(norm_q, "norm_q", torch.float32, True), _ptr(norm_k, "norm_k", torch.float32, True), float(eps),
         _ptr(q_out, "q_out", dt), _ptr(k_pages, "k_pages", dt, not write_kv), _ptr(v_pages, "v_pages", dt, not write_kv),
         _ptr(positions, "positions", torch.int32), _ptr(slot_map, "slot_map", torch.int32) if write_kv else None,
-        _ptr(inv_freq, "inv_freq", torch.float32, True), int(rot), _ptr(inv_freq_v, "inv_freq_v", torch.float32, True),
+        _ptr(inv_freq, "inv_freq", torch.float32, True), int(rot), float(rot_magnitude),
+        _ptr(inv_freq_v, "inv_freq_v", torch.float32, True),
         T, HQ, GK, GV, D, Vd, page_size, int(bool(k_tiled)), int(bool(v_tiled)), Dp, _stream()), "qkv_prepare")
 
 
 def attn_wide(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T, HQ, GK, GV, D, Vd, page_size, vis, span,
-              scale, k_tiled=False, v_tiled=False):
+              scale, k_tiled=False, v_tiled=False, sinks=None):
     """Attention over the paged cache with keys of D and values of Vd elements, HQ query heads over
     GK key heads over GV value heads (query head h: key head h // (HQ/GK), value head of that % GV);
-    any mix of portions and single tokens.  q [T, HQ*D]; out [T, HQ*Vd] in q's dtype or fp32."""
+    any mix of portions and single tokens.  q [T, HQ*D]; out [T, HQ*Vd] in q's dtype or fp32.
+    ``sinks`` (fp32 [HQ] or None): one more term exp(sinks[h]) in every softmax's denominator."""
+    if sinks is not None and sinks.numel() != HQ:
+        raise KernelError(f"attention: {sinks.numel()} sinks for {HQ} query heads")
     if q.numel() < T * HQ * D or out.numel() < T * HQ * Vd:
         raise KernelError("attention: q or out too small")
     if tuple(k_pages.shape[1:]) != (GK, page_size, D) or tuple(v_pages.shape[1:]) != (GV, Vd, page_size) \
@@ -828,7 +847,8 @@ def attn_wide(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T,
         _ptr(q, "q"), _ptr(k_pages, "k_pages", dt), _ptr(v_pages, "v_pages", dt), _ptr(out, "out"), dtype_code(dt),
         dtype_code(out.dtype), _ptr(positions, "positions", torch.int32), _ptr(seq_of_token, "seq_of_token", torch.int32),
         _ptr(block_table, "block_table", torch.int32), block_table.shape[1], T, HQ, GK, GV, D, Vd, page_size,
-        VIS[vis], int(span or 0), float(scale), int(bool(k_tiled)), int(bool(v_tiled)), _stream()), "attention")
+        VIS[vis], int(span or 0), float(scale), int(bool(k_tiled)), int(bool(v_tiled)),
+        _ptr(sinks, "sinks", torch.float32, True), _stream()), "attention")
 
 
 def attn_finish(a, out, positions, H, Vd, *, maps=1, lam=0.0, eps=0.0, post=1.0, inv_freq_v=None, gate=None):
@@ -873,3 +893,77 @@ def act_rows(x, act):
     if act not in UNARY_ACTS:
         raise KernelError(f"act_rows: activation {act!r} (known: {sorted(UNARY_ACTS)})")
     _check(lib().spite_act_rows(_ptr(x, "x"), dtype_code(x.dtype), x.numel(), UNARY_ACTS[act], _stream()), "act_rows")
+
+
+def scale_rows(x, c: float):
+    """x *= c in place; x fp32."""
+    _check(lib().spite_scale_rows(_ptr(x, "x", torch.float32), x.numel(), float(c), _stream()), "scale_rows")
+
+
+# -------------------------------------------------------------------------------------------- linear attention
+def channel_decay(z, bias, tau: float):
+    """z[t, c] = sigmoid(z[t, c] + bias[c]) ** (1 / tau) in place; z fp32 [T, n], bias fp32 [n] or None."""
+    T, n = z.shape
+    if bias is not None and bias.numel() != n:
+        raise KernelError(f"channel_decay: bias of {bias.numel()} for rows of {n}")
+    if not tau > 0:
+        raise KernelError(f"channel_decay: tau = {tau}")
+    _check(lib().spite_channel_decay(_ptr(z, "z", torch.float32), _ptr(bias, "bias", torch.float32, True), T, n,
+                                     1.0 / float(tau), _stream()), "channel_decay")
+
+
+def _rows_view(t, name, width, T):
+    """Pointer and row stride of a [T, >= width] view whose rows may lie apart."""
+    if t.dim() != 2 or t.stride(1) != 1 or t.shape[0] < T or t.shape[1] < width or not t.is_cuda:
+        raise KernelError(f"{name}: {tuple(t.shape)} with strides {t.stride()} for {T} rows of {width}")
+    return t.data_ptr(), t.stride(0)
+
+
+def linear_attn_scan(q, k, v, out, state, cu_seqlens, seq_slots, n_seqs, H, D, V, *, decay=None, head_decay=None,
+                     q_scale=1.0, keep=True):
+    """The recurrence S = diag(a) S + k v^T, o = S^T q token by token for every entry of the step (see
+    linear_attn.hip).  q, k [T, H*D] and v [T, H*V]: views of the run's dtype whose rows may lie apart;
+    ``decay`` fp32 [T, H*D] (a number per key channel and token) or ``head_decay`` fp32 [H]; ``state`` fp32
+    [slots, H, D, V], read at the entry's slot and, with ``keep``, left as the entry's last token leaves it;
+    out fp32 [T, H*V]."""
+    T = out.shape[0]
+    if q.dtype != k.dtype or q.dtype != v.dtype:
+        raise KernelError("linear_attn_scan: q, k and v of one dtype")
+    pq, ldq = _rows_view(q, "q", H * D, T)
+    pk, ldk = _rows_view(k, "k", H * D, T)
+    pv, ldv = _rows_view(v, "v", H * V, T)
+    if out.numel() < T * H * V or tuple(state.shape[1:]) != (H, D, V):
+        raise KernelError(f"linear_attn_scan: out {tuple(out.shape)}, state {tuple(state.shape)} for H={H} D={D} V={V}")
+    if decay is not None and decay.numel() < T * H * D:
+        raise KernelError("linear_attn_scan: decay too small")
+    if head_decay is not None and head_decay.numel() != H:
+        raise KernelError(f"linear_attn_scan: {head_decay.numel()} decays for {H} heads")
+    if cu_seqlens.numel() < n_seqs + 1 or seq_slots.numel() < n_seqs:
+        raise KernelError("linear_attn_scan: metadata too small")
+    _check(lib().spite_linear_attn_scan(
+        pq, pk, pv, ldq, ldk, ldv, dtype_code(q.dtype), _ptr(decay, "decay", torch.float32, True),
+        _ptr(head_decay, "head_decay", torch.float32, True), float(q_scale), _ptr(state, "state", torch.float32),
+        state.shape[0], _ptr(cu_seqlens, "cu_seqlens", torch.int32), _ptr(seq_slots, "seq_slots", torch.int32), int(n_seqs),
+        _ptr(out, "out", torch.float32), H, D, V, int(bool(keep)), _stream()), "linear_attn_scan")
+
+
+NORM_GATES = {None: 0, "silu": 1, "sigmoid": 2}
+
+
+def gated_group_norm(o, weight, y, group, eps, gate=None, act=None):
+    """y = rmsnorm(o over groups of ``group`` elements) * weight * act(gate).  o fp32 [T, n]; weight fp32
+    of ``group`` elements (shared by the groups) or of n; gate a [T, n] view in y's dtype (rows may lie
+    apart) with ``act`` silu or sigmoid, or None; y [T, n]."""
+    T, n = o.shape
+    if act not in NORM_GATES or (act is None) != (gate is None):
+        raise KernelError(f"gated_group_norm: gate activation {act!r} (known: silu, sigmoid) with a gate, or neither")
+    pg, ldg = (None, 0)
+    if gate is not None:
+        if gate.dtype != y.dtype:
+            raise KernelError("gated_group_norm: the gate has the output's dtype")
+        pg, ldg = _rows_view(gate, "gate", n, T)
+    if y.numel() < T * n:
+        raise KernelError("gated_group_norm: output too small")
+    _check(lib().spite_gated_group_norm(_ptr(o, "o", torch.float32), pg, ldg, _ptr(weight, "weight", torch.float32),
+                                        weight.numel(), _ptr(y, "y"), dtype_code(y.dtype), T, n, int(group), float(eps),
+                                        NORM_GATES[act], _stream()), "gated_group_norm")

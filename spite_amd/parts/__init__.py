@@ -2,4 +2,4 @@
 from .base import (ParamSpec, KVNeed, StateNeed, CacheNeed, PartSpec, BlockSpec, LayerCall, ModelSpec,
                    Part, Norm, PositionEncoding, Mixer, FeedForward, Block, Embedding, Head, SideInput, InputShift, register, build,
                    registered, UnknownPart, two_increments, NormedIncrement)
-from . import norm, position, attention, latent_attention, wide_attention, feed_forward, side, shift, block, ends  # noqa: F401  (registration)
+from . import norm, position, attention, latent_attention, wide_attention, linear_attention, feed_forward, side, shift, block, ends  # noqa: F401  (registration)

@@ -68,6 +68,8 @@ class Attention(Mixer):
         self.temperature = temperature            # None or (floor_scale, attn_scale)
         self.scale = float(softmax_scale) if softmax_scale is not None else 1.0 / math.sqrt(self.hd)
         self.position = build_part("position", position, env)
+        if self.position.kernel_args().get("magnitude", 1.0) != 1.0:
+            raise ValueError("attention: a position encoding that scales sine and cosine is not what this mixer's kernel applies")
         self.graph_safe = self.position.graph_safe
         self.wqkv = self.wo = self.slopes = None
 

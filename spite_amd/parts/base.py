@@ -23,6 +23,9 @@ class ParamSpec:
     shape: Tuple[int, ...]
     kind: str = "matrix"    # "matrix": computed in the run's dtype; "vector": always fp32; "int": int32
     init: str = "normal"    # random-weights mode: "normal" N(0,std), "ones" 1+N(0,std), "zeros"
+    free: Tuple[int, ...] = ()   # axes whose size the checkpoint decides (an inner width that no configuration key
+                                 # names); ``shape`` holds what random weights are drawn with there, and the part
+                                 # reads the true size off the tensors it is handed (``load``)
 
 
 @dataclass(frozen=True)

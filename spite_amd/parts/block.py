@@ -154,11 +154,13 @@ class SandwichBlock(Block):
 
 @register("block", "parallel")
 class ParallelBlock(Block):
-    """Mixer and feed-forward read the same stream, each through a norm of its own, and their
-    results join it together:  h += mixer(shift(norm1(h))) + ffn(norm2(h)).  ``spec.extra["shift"]``
-    (a PartSpec of category ``shift``, optional) stands between the first norm and the mixer and
-    keeps a state row per request; the feed-forward may be missing.  Both results are handed to the
-    next block, whose first norm adds them."""
+    """Mixer and feed-forward read the same stream and their results join it together:
+    h += mixer(shift(norm1(h))) + ffn(norm2(h)), each through a norm of its own, or, where the spec
+    names no second norm, both through the one norm: h += mixer(n) + ffn(n), n = norm1(h).
+    ``spec.extra["shift"]`` (a PartSpec of category ``shift``, optional) stands between the first norm
+    and the mixer and keeps a state row per request; the feed-forward may be missing;
+    ``spec.extra["side"]`` (category ``side``, optional) adds its input from the step's tokens to the
+    stream after both.  The results are handed to the next block, whose first norm adds them."""
     graph_safe = True
 
     def __init__(self, env, spec):
@@ -166,15 +168,20 @@ class ParallelBlock(Block):
         self.norm1 = build_part("norm", spec.norm1, env)
         self.mixer = build_part("mixer", spec.mixer, env)
         self.children = [("norm1", self.norm1, spec.norm1), ("mixer", self.mixer, spec.mixer)]
-        self.shift = self.norm2 = self.ffn = None
+        self.shift = self.norm2 = self.ffn = self.side = None
         sh = spec.extra.get("shift")
         if sh is not None:
             self.shift = build_part("shift", sh, env)
             self.children.append(("shift", self.shift, sh))
         if spec.ffn is not None:
-            self.norm2 = build_part("norm", spec.norm2, env)
+            if spec.norm2 is not None:
+                self.norm2 = build_part("norm", spec.norm2, env)
+                self.children.append(("norm2", self.norm2, spec.norm2))
             self.ffn = build_part("ffn", spec.ffn, env)
-            self.children += [("norm2", self.norm2, spec.norm2), ("ffn", self.ffn, spec.ffn)]
+            self.children.append(("ffn", self.ffn, spec.ffn))
+        if spec.extra.get("side") is not None:
+            self.side = build_part("side", spec.extra["side"], env)
+            self.children.append(("side", self.side, spec.extra["side"]))
         self.children = tuple(self.children)
         self.graph_safe = all(part.graph_safe for _, part, _ in self.children)
         self.step_arrays = tuple(sorted({a for _, part, _ in self.children for a in part.step_arrays}))
@@ -194,13 +201,17 @@ class ParallelBlock(Block):
 
     def stages(self):
         first = all(p.graph_safe for p in (self.norm1, self.shift, self.norm2) if p is not None)
-        return [(first, self._stage_norms), (self.mixer.graph_safe, self._stage_mixer),
-                (self.ffn is None or self.ffn.graph_safe, self._stage_ffn)]
+        last = all(p.graph_safe for p in (self.ffn, self.side) if p is not None)
+        return [(first, self._stage_norms), (self.mixer.graph_safe, self._stage_mixer), (last, self._stage_ffn)]
 
     def _stage_norms(self, state, ctx, cache):
         h, ws = state["h"], ctx.ws
         T, d = h.shape
-        d1, d2 = two_increments(h, state["pending"])
+        d1, d2, normed = SandwichBlock._split(h, state["pending"])
+        extra = {} if normed is None else {"normed": normed}
+        if self.ffn is not None and self.norm2 is None:
+            self._one_norm(state, ctx, cache, d1, d2, extra)
+            return
         n2 = n2_32 = None
         if self.ffn is not None:
             n2 = ws.take((T, d), self.env.dtype)
@@ -212,18 +223,41 @@ class ParallelBlock(Block):
         if self.shift is not None:
             # the shift blends fp32 rows; the mixer's input takes the run's dtype after it
             n32 = ws.take((T, d), torch.float32)
-            self.norm1.forward(h, None, d1=d1, d2=d2, out32=n32, **both)
+            self.norm1.forward(h, None, d1=d1, d2=d2, out32=n32, **both, **extra)
             x = ws.take((T, d), self.env.dtype)
             self.shift.forward(n32, x, ctx, cache["shift"].state)        # a block with a shift has two caches, by name
         else:
             x = ws.take((T, d), self.env.dtype)
-            self.norm1.forward(h, x, d1=d1, d2=d2, **both)
+            self.norm1.forward(h, x, d1=d1, d2=d2, **both, **extra)
         state["mixer_in"] = x
         if self.ffn is not None:
             if not paired:
                 # the same stream (the increments are in it now) through the second norm
                 self.norm2.forward(h, n2, out32=None if n2_32 is n2 else n2_32, write_h=False)
-            state["ffn_in"] = (n2, n2_32)
+            state["ffn_in"] = (n2, n2_32, None)
+
+    def _one_norm(self, state, ctx, cache, d1, d2, extra):
+        """One norm for both sublayers: its rows are the feed-forward's input and (through the shift, if
+        there is one) the mixer's; the feed-forward's small fp32 products (router logits) are formed in the
+        same pass where the norm can do that."""
+        h, ws = state["h"], ctx.ws
+        T, d = h.shape
+        n = ws.take((T, d), self.env.dtype)
+        proj = self.ffn.input_projection()
+        n32 = logits = None
+        if self.shift is not None or (self.ffn.wants_f32_input and not (proj is not None and self.norm1.can_project(proj))):
+            n32 = n if n.dtype == torch.float32 and self.shift is None else ws.take((T, d), torch.float32)
+        if proj is not None and self.norm1.can_project(proj):
+            logits = ws.take((T, proj.shape[0]), torch.float32)
+            self.norm1.forward(h, n, d1=d1, d2=d2, out32=None if n32 is n else n32, proj=proj, proj_out=logits, **extra)
+        else:
+            self.norm1.forward(h, n, d1=d1, d2=d2, out32=None if n32 is n else n32, **extra)
+        x = n
+        if self.shift is not None:
+            x = ws.take((T, d), self.env.dtype)
+            self.shift.forward(n32, x, ctx, cache["shift"].state)
+        state["mixer_in"] = x
+        state["ffn_in"] = (n, n32 if self.ffn.wants_f32_input and logits is None else None, logits)
 
     def _stage_mixer(self, state, ctx, cache):
         state["mixed"] = self.mixer.forward(state.pop("mixer_in"), ctx, cache["mixer"] if isinstance(cache, dict) else cache)
@@ -231,6 +265,11 @@ class ParallelBlock(Block):
     def _stage_ffn(self, state, ctx, cache):
         pend = (state.pop("mixed"),)
         if self.ffn is not None:
-            n2, n2_32 = state.pop("ffn_in")
-            pend += tuple(self.ffn.forward(n2, n2_32, ctx))
+            n2, n2_32, logits = state.pop("ffn_in")
+            if logits is not None:
+                pend += tuple(self.ffn.forward(n2, None, ctx, projected=logits))
+            else:
+                pend += tuple(self.ffn.forward(n2, n2_32, ctx))
+        if self.side is not None:
+            pend = tuple(self.side.forward(state["h"], pend, ctx))
         state["pending"] = pend

@@ -3,7 +3,7 @@
 ``token_table`` (crates/spite-models/src/llama/llama4.rs:118-119): row ``id`` of the table as
 the residual stream's first value, in fp32, times ``scale`` if the architecture has one.
 ``linear_head`` (llama4.rs:277-279): logits = W . (normed last hidden state), W ``[V, d]``;
-tied, it reads the embedding's table.  Another architecture's embedding scale, logit cap or
+tied, it reads the embedding's table; times ``scale`` if the architecture has one.  Another architecture's embedding scale, logit cap or
 bias is another kind registered under these categories, not a change to the model class.
 """
 from __future__ import annotations
@@ -36,8 +36,9 @@ class TokenTable(Embedding):
 class LinearHead(Head):
     graph_safe = True
 
-    def __init__(self, env, vocab_size: int, width: int, tied: bool = False):
-        self.V, self.d, self.tied = int(vocab_size), int(width), bool(tied)
+    def __init__(self, env, vocab_size: int, width: int, tied: bool = False, scale: float = 1.0):
+        """``scale``: a constant on the logits (fp32)."""
+        self.V, self.d, self.tied, self.scale = int(vocab_size), int(width), bool(tied), float(scale)
         self.weight = None
 
     def params(self):
@@ -57,3 +58,5 @@ class LinearHead(Head):
 
     def forward(self, x, logits, ctx):
         linear(x, self.weight, logits, ws=ctx.ws)
+        if self.scale != 1.0:
+            hipops.scale_rows(logits, self.scale)

@@ -1,7 +1,8 @@
 """Feed-forward parts.
 
 ``dense_glu`` (crates/spite-models/src/llama/llama4.rs:257-271):
-y = W_down . (silu(W_gate . x) * (W_up . x)).
+y = W_down . (act(W_gate . x) * (W_up . x)), act = silu there; ``gelu_tanh`` and ``relu`` are the
+gate's other activations.
 
 ``dense_mlp``: y = W_down . act(W_up . x), no gate; ``activation``: ``gelu`` (the erf form),
 ``gelu_tanh`` or ``silu``, applied in fp32 to the up projection's rows.
@@ -19,6 +20,9 @@ the largest s + bias (a per-expert correction that steers the choice only); each
 expert of its own width may run for every token.  The choices of a step are ``top_k`` entries a
 token; the expert plan sorts them by expert, the grouped products walk that list, every entry
 gets an output row of its own and a last kernel forms the weighted sum per token.
+
+``moe_topk_softmax``: the same part with the other way of scoring: the ``top_k`` experts with the largest
+logits are taken and their weights are the softmax over the taken logits alone; no bias.
 """
 from __future__ import annotations
 
@@ -36,10 +40,10 @@ class DenseGLU(FeedForward):
     graph_safe = True
 
     def __init__(self, env, hidden_size, intermediate_size, activation="silu"):
-        """``activation``: the gate's, ``silu`` or ``gelu_tanh``."""
+        """``activation``: the gate's, ``silu``, ``gelu_tanh`` or ``relu``."""
         self.d, self.F = int(hidden_size), int(intermediate_size)
         if hipops.GATE_ACTS.get(activation, 0) == 0:
-            raise ValueError(f"dense_glu: activation {activation!r} (known: silu, gelu_tanh)")
+            raise ValueError(f"dense_glu: activation {activation!r} (known: silu, gelu_tanh, relu)")
         self.activation = activation
         self.w_gate_up = self.w_down = None
 
@@ -212,13 +216,18 @@ class MoeTopKSigmoid(FeedForward):
     wants_f32_input = True
 
     def __init__(self, env, hidden_size, intermediate_size, n_experts, top_k, shared_intermediate_size=None,
-                 score_bias=True, renormalize=False, activation="silu"):
+                 score_bias=True, renormalize=False, activation="silu", scoring="sigmoid"):
+        """``scoring``: ``sigmoid`` (the choice by sigmoid(z) + bias, weights sigmoid(z)) or ``softmax_taken`` (the
+        choice by z + bias, weights the softmax over the taken experts' z)."""
+        if scoring not in hipops.ROUTER_SCORING:
+            raise ValueError(f"moe: scoring {scoring!r} (known: {sorted(hipops.ROUTER_SCORING)})")
+        self.scoring = scoring
         self.d, self.F, self.E, self.k = int(hidden_size), int(intermediate_size), int(n_experts), int(top_k)
         self.Fs = None if shared_intermediate_size is None else int(shared_intermediate_size)
         if not 1 <= self.k <= self.E or self.E > 512:
             raise ValueError(f"moe: {self.k} of {self.E} experts (at most 512)")
         if hipops.GATE_ACTS.get(activation, 0) == 0:
-            raise ValueError(f"moe: activation {activation!r} (known: silu, gelu_tanh)")
+            raise ValueError(f"moe: activation {activation!r} (known: silu, gelu_tanh, relu)")
         self.score_bias, self.renormalize, self.activation = bool(score_bias), bool(renormalize), activation
         self.w_router = self.bias = self.w_gate_up = self.w_down = self.ws_gate_up = self.ws_down = None
 
@@ -274,7 +283,7 @@ class MoeTopKSigmoid(FeedForward):
             take = trace["take_experts"].pop(0).to(device=x.device, dtype=torch.int64).view(T, k)
             logits = torch.full_like(logits, float("-inf")).scatter_(1, take, logits.gather(1, take))
             bias = None
-        hipops.router_topk(logits, bias, expert, weight, k, renorm=self.renormalize)
+        hipops.router_topk(logits, bias, expert, weight, k, renorm=self.renormalize, scoring=self.scoring)
         if trace is not None:                         # a testing aid: which experts each token took, [T, top_k]
             trace.setdefault("moe_experts", []).append(expert.view(T, k).clone())
         src, dst, unused = ws.take((n,), torch.int32), ws.take((n,), torch.int32), ws.take((n,), torch.float32)
@@ -296,3 +305,13 @@ class MoeTopKSigmoid(FeedForward):
         out = ws.take((T, d), torch.float32)
         hipops.moe_combine(y, weight, ys, out, T, k)
         return (out,)
+
+
+@register("ffn", "moe_topk_softmax")
+class MoeTopKSoftmax(MoeTopKSigmoid):
+    """Several experts a token, taken by their logits and weighted by the softmax over the taken ones."""
+
+    def __init__(self, env, hidden_size, intermediate_size, n_experts, top_k, shared_intermediate_size=None,
+                 activation="silu"):
+        super().__init__(env, hidden_size, intermediate_size, n_experts, top_k, shared_intermediate_size,
+                         score_bias=False, renormalize=False, activation=activation, scoring="softmax_taken")

@@ -57,6 +57,8 @@ class LatentAttention(Mixer):
         self.cache_span = int(cache_span if cache_span is not None else self.span)
         self.own = bool(own_kv)
         self.position = build_part("position", position, env)
+        if self.position.kernel_args().get("magnitude", 1.0) != 1.0:
+            raise ValueError("latent_attention: a position encoding that scales sine and cosine is not what this mixer's kernel applies")
         ka = self.position.kernel_args()
         if self.r and not (ka.get("use_rope") and ka.get("adjacent")):
             raise ValueError("latent attention: the rotated parts take a rotary encoding with adjacent pairs")

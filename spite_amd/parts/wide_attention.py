@@ -16,7 +16,10 @@ keys and queries ``key_dim`` wide, values ``value_dim`` wide, with, each as an o
   head's values, times ``1 - diff``; lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff is one number
   of the layer, formed from four vectors of the checkpoint when it is loaded;
 * ``head_gate``: head h's result times sigmoid(W_g x)_h (``gate_proj`` [H, d]), before the output
-  projection.
+  projection;
+* ``sinks``: every head's softmax has one more term in its denominator, exp(s_h) with a learned number
+  s_h per head (``sink`` [H]): it is no key, is not scaled, brings no value and counts once, so a head
+  may give less than all of its weight to the keys it sees.
 
 Inside, two maps are 2H query heads over 2G key heads over G value heads: the projections' rows
 are reordered map by map when they are loaded, so that query head m*H + h reads key head
@@ -42,7 +45,7 @@ class WideAttention(Mixer):
 
     def __init__(self, env, hidden_size, n_heads, n_kv_heads, key_dim, value_dim, scale, position=None,
                  value_position=None, visibility="full", span=0, bias=False, projection_norm=False, norm_eps=1e-5,
-                 maps=1, diff=0.0, head_gate=False):
+                 maps=1, diff=0.0, head_gate=False, sinks=False):
         if n_heads % n_kv_heads:
             raise ValueError(f"wide_attention: {n_heads} heads over {n_kv_heads} kv heads")
         if visibility not in hipops.VIS:
@@ -51,14 +54,16 @@ class WideAttention(Mixer):
             raise ValueError(f"wide_attention: {visibility} of size {span}")
         if maps not in (1, 2):
             raise ValueError(f"wide_attention: {maps} score maps a head")
-        if maps == 2 and (value_position is not None or head_gate):
-            raise ValueError("wide_attention: two score maps go with neither turned values nor a head gate")
+        if maps == 2 and (value_position is not None or head_gate or sinks):
+            raise ValueError("wide_attention: two score maps go with neither turned values nor a head gate nor sinks")
         self.env = env
         self.d, self.H, self.G = int(hidden_size), int(n_heads), int(n_kv_heads)
         self.D, self.Vd, self.maps = int(key_dim), int(value_dim), int(maps)
         self.scale, self.diff, self.eps = float(scale), float(diff), float(norm_eps)
         self.visibility, self.span = visibility, int(span or 0)
         self.bias, self.projection_norm, self.head_gate = bool(bias), bool(projection_norm), bool(head_gate)
+        self.sinks = bool(sinks)
+        self.w_sink = None
         self.position = build_part("position", position, env) if position is not None else None
         self.value_position = build_part("position", value_position, env) if value_position is not None else None
         for pe in (self.position, self.value_position):
@@ -74,6 +79,7 @@ class WideAttention(Mixer):
         self.w_in = self.wo = self.b_in = self.w_qnorm = self.w_knorm = None
         self.inv_freq = self.inv_freq_v = None
         self.rot = 0
+        self.rot_magnitude = 1.0
         self.lam = 0.0
 
     # ------------------------------------------------------------------ tensors
@@ -92,6 +98,8 @@ class WideAttention(Mixer):
             p.update({k: ParamSpec((D,), kind="vector", init="normal") for k in ("lambda_q1", "lambda_k1", "lambda_q2", "lambda_k2")})
         if self.head_gate:
             p["gate_proj"] = ParamSpec((H, d))
+        if self.sinks:
+            p["sink"] = ParamSpec((H,), kind="vector", init="normal")
         return p
 
     def _by_map(self, t, heads):
@@ -122,16 +130,19 @@ class WideAttention(Mixer):
         if self.maps == 2:
             dot = lambda a, b: float((t[a].double() * t[b].double()).sum())
             self.lam = math.exp(dot("lambda_q1", "lambda_k1")) - math.exp(dot("lambda_q2", "lambda_k2")) + self.diff
+        if self.sinks:
+            self.w_sink = t["sink"].float().contiguous()
         if self.position is not None:
             ka = self.position.kernel_args()
             if ka["use_rope"]:
                 self.inv_freq, self.rot = ka["inv_freq"], int(ka.get("rotary_dim") or self.D)
+                self.rot_magnitude = float(ka.get("magnitude", 1.0))
                 if self.rot > self.D:
                     raise ValueError(f"wide_attention: {self.rot} turning elements in heads of {self.D}")
         if self.value_position is not None:
             ka = self.value_position.kernel_args()
-            if int(ka.get("rotary_dim") or self.Vd) != self.Vd or self.Vd % 2:
-                raise ValueError("wide_attention: the values' rotation covers the whole (even) value width")
+            if int(ka.get("rotary_dim") or self.Vd) != self.Vd or self.Vd % 2 or ka.get("magnitude", 1.0) != 1.0:
+                raise ValueError("wide_attention: the values' rotation is a pure one over the whole (even) value width")
             self.inv_freq_v = ka["inv_freq"]
 
     def slow_paths(self, page_size):
@@ -164,7 +175,7 @@ class WideAttention(Mixer):
         scratch = ctx.ws.take((hipops.attn_decode_workspace(T, HQ, D, n_splits) // 4,), torch.float32)
         hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
                            cache.block_table, T, HQ, GK, D, cache.page_size, self.visibility, self.span,
-                           self.scale, n_splits, value_heads=self.G)
+                           self.scale, n_splits, value_heads=self.G, sinks=self.w_sink)
 
     def _prefill(self, q, o, ctx, cache, lead, cu_seqlens):
         HQ, GK, D = self.HQ, self.GK, self.Dk
@@ -178,7 +189,7 @@ class WideAttention(Mixer):
             scratch = ctx.ws.take((hipops.attn_prefill_workspace(counts, HQ, GK, D, n_splits) // 4,), torch.float32)
         hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions[lead:], cu_seqlens, counts,
                             cache.block_table[lead:], HQ, GK, D, cache.page_size, self.visibility, self.span, self.scale,
-                            n_splits=n_splits, scratch=scratch, value_heads=self.G)
+                            n_splits=n_splits, scratch=scratch, value_heads=self.G, sinks=self.w_sink)
 
     def forward(self, x, ctx, cache):
         T, ws = x.shape[0], ctx.ws
@@ -189,7 +200,7 @@ class WideAttention(Mixer):
         hipops.qkv_prepare(proj, q, cache.k_pages, cache.v_pages, ctx.positions, cache.slot_map, HQ, GK, G, D, Vd,
                            cache.page_size, bias=self.b_in, norm_q=self.w_qnorm, norm_k=self.w_knorm, eps=self.eps,
                            inv_freq=self.inv_freq, rot=self.rot, inv_freq_v=self.inv_freq_v, write_kv=cache.write,
-                           k_tiled=cache.tiled, v_tiled=cache.tiled, stored_dim=Dk)
+                           k_tiled=cache.tiled, v_tiled=cache.tiled, stored_dim=Dk, rot_magnitude=self.rot_magnitude)
         if cache.tiled and self._mfma(cache.page_size):
             a = ws.take((T, HQ * Vd), x.dtype)
             cu_tail, lead = ctx.derived[TAIL]
@@ -204,7 +215,7 @@ class WideAttention(Mixer):
             a = ws.take((T, HQ * Vd), torch.float32 if self.maps == 2 else x.dtype)
             hipops.attn_wide(q, cache.k_pages, cache.v_pages, a, ctx.positions, ctx.seq_of_token, cache.block_table,
                              T, HQ, GK, G, Dk, Vd, cache.page_size, self.visibility, self.span, self.scale,
-                             k_tiled=cache.tiled, v_tiled=cache.tiled)
+                             k_tiled=cache.tiled, v_tiled=cache.tiled, sinks=self.w_sink)
         if self.maps == 2 or self.inv_freq_v is not None or self.head_gate:
             o = ws.take((T, H * Vd), x.dtype)
             gate = proj[:, self.n_qkv:self.n_qkv + H] if self.head_gate else None

@@ -148,8 +148,9 @@ def bind(model, source, checkpoint_dtype: torch.dtype = torch.bfloat16) -> None:
         if n not in have:
             continue
         dt, shape = source.info(n)
-        if tuple(shape) != tuple(ps.shape):
-            shapes.append((n, shape, ps.shape))
+        free = set(getattr(ps, "free", ()))
+        if len(shape) != len(ps.shape) or any(a != e and ax not in free for ax, (a, e) in enumerate(zip(shape, ps.shape))):
+            shapes.append((n, shape, tuple("any" if ax in free else e for ax, e in enumerate(ps.shape))))
         is_int = not dt.is_floating_point
         if (ps.kind == "int") != is_int:
             kinds.append((n, dt, "an integer type" if ps.kind == "int" else "a floating type"))
