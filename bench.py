@@ -223,6 +223,11 @@ class KernelTimes:
 # (half as many heads, two score maps of 64 each over values of 128: the same score and value products a
 # token as the other layers), a window of 4,096 everywhere, an ungated feed-forward 1.5 times as wide as
 # Llama 4's gated one (``dense_ff``), so that both have the same products a token.
+# ``--design tebalorn``: the Tebalorn design beside Llama 4 with the same experts.  Tebalorn: layers in the order
+# gla, lightning, attention, lightning (linear attention with heads of 128 key channels and 128 values, a state of
+# heads x 128 x 128 numbers a request; softmax attention with sinks, heads of 128, a kv head for every four, the first
+# 64 elements turning with YaRN-scaled frequencies, chunks of 4,096), every layer with the experts of the size, their
+# shared expert and per-layer token rows of 256.
 DESIGN_SIZES = {
     "2k": dict(width=2048, heads=16, experts=16, top=4, expert_ff=1024, shared_ff=2048, dense_ff=8192),
     "5k": dict(width=5120, heads=40, experts=16, top=2, expert_ff=4096, shared_ff=8192, dense_ff=16384),
@@ -247,9 +252,33 @@ def pefedra_configs(sz, layers, window, vocab):
     return {"pefedra": pefedra, "llama4": llama}
 
 
+def tebalorn_configs(sz, layers, window, vocab):
+    H = sz["heads"]
+    linear = {"heads": H, "dim": 128, "vdim": 128}
+    mixers = [("gla", dict(linear, tau=16.0)),
+              ("lightning", dict(linear, decay=[1.0 - 2.0 ** (-5.0 - 3.0 * h / max(H - 1, 1)) for h in range(H)])),
+              ("attention", {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                             "mask": {"size": window},
+                             "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}),
+              ("lightning", dict(linear, decay=[1.0 - 2.0 ** (-4.0 - 4.0 * h / max(H - 1, 1)) for h in range(H)]))]
+    mlp = {"kind": "moe", "router": {"experts": sz["experts"], "top": sz["top"]}, "expert": {"ff": sz["expert_ff"]},
+           "shared": {"ff": sz["shared_ff"]}}
+    tebalorn = {"architecture": "Tebalorn", "vocab": vocab, "width": sz["width"], "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+                "logit_scale": 0.5, "token_side": {"dim": 256}, "torch_dtype": "bfloat16",
+                "layers": [{"type": mixers[i % 4][0], "mixer": mixers[i % 4][1], "mlp": mlp} for i in range(layers)]}
+    each = (sz["top"] * sz["expert_ff"] + sz["shared_ff"]) // 2
+    llama = dict(SCOUT, num_hidden_layers=layers, hidden_size=sz["width"], num_attention_heads=H,
+                 num_key_value_heads=max(1, H // 4), head_dim=128, num_local_experts=sz["experts"],
+                 intermediate_size=each, intermediate_size_mlp=2 * each, vocab_size=vocab, attention_chunk_size=window,
+                 no_rope_layers=None, rope_scaling=None)
+    return {"tebalorn": tebalorn, "llama4": llama}
+
+
 def design_configs(sz, layers, window, vocab, design="ravenex"):
     if design == "pefedra":
         return pefedra_configs(sz, layers, window, vocab)
+    if design == "tebalorn":
+        return tebalorn_configs(sz, layers, window, vocab)
     mix = lambda kv_from: dict({"heads": sz["heads"], "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
                                 "mask": {"size": window}, "rot": {"base": 10000.0, "dims": 64}, "scale": 192 ** -0.5},
                                **({} if kv_from is None else {"kv_from": kv_from}))
@@ -606,7 +635,7 @@ def main() -> int:
     ap.add_argument("--workload", default="decode", choices=["decode", "longctx", "serve", "designs"],
                     help="designs: another design (--design) beside Llama 4 at equal sizes (see DESIGN_SIZES)")
     ap.add_argument("--design-sizes", default="2k,5k", help="designs: which of DESIGN_SIZES, comma separated")
-    ap.add_argument("--design", default="ravenex", choices=["ravenex", "pefedra"],
+    ap.add_argument("--design", default="ravenex", choices=["ravenex", "pefedra", "tebalorn"],
                     help="designs: which design runs beside Llama 4 (pefedra: against Llama 4 with dense layers only)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (memory or time)")
     ap.add_argument("--batch", type=int, default=8)
