@@ -8,8 +8,8 @@
 // [slots, H, D, V]; every sum and product of the recurrence is fp32 whatever the type of q, k and v.
 //
 // channel_decay:      z -> sigmoid(z + b)^(1/tau) in place, through its logarithm.
-// linear_attn_scan:   the recurrence token by token: the plain form, whose bits do not depend on how a
-//                     request's tokens are cut into steps.
+// linear_attn_scan:   the recurrence token by token, in fp32 FMAs, with the tokens' rows staged through LDS in
+//                     blocks; its bits do not depend on how a request's tokens are cut into steps.
 // gated_group_norm:   y = rmsnorm(o over groups of `group` elements) * w * act(gate), the step between the
 //                     recurrence and the output projection.
 #include "common.h"
@@ -39,87 +39,154 @@ extern "C" int spite_channel_decay(float* z, const float* bias, int T, int width
 // ------------------------------------------------------------------ the recurrence, token by token
 // A workgroup of 256 threads takes 16 value columns of one head of one entry of the step and walks the
 // entry's tokens in order.  Thread (vc, dg) = (tid / 16, tid % 16) holds the state's elements
-// S[dg + 16 r][v0 + vc], r < ceil(D / 16), in registers.  A token's q, k and decay go through LDS (two
-// buffers: the next token's are on their way while this one is computed, one barrier a token); the
-// sum over the key channels is a thread's own partial sum and four steps across its 16 neighbours.
-// The order of every sum is fixed by D alone.
+// S[dg * RR + r][v0 + vc], r < RR (RR = 4, 8 or 16 for up to 64, 128 or 256 key channels), in registers.
+// The tokens' q, k, decay and value slice go through LDS a block of LA_TB tokens at a time, two buffers:
+// the next block's loads are in flight while this block is computed, so a token costs its FMAs, a few
+// wide LDS reads and four steps across the thread's 16 neighbours, and one barrier a block.  The
+// dependent chain from token to token is the one FMA of the state.  The state tile goes through LDS on
+// the way in and out, so that its rows are read and written 64 bytes at a time.
+// The order of every sum is fixed by D alone: the bits do not depend on how a request's tokens are cut.
 #define LA_VC 16
 #define LA_DG 16
-#define LA_MAXR 16       // key channels up to 256
+#define LA_MAXD 256
 
-template <typename T>
+template <int RR> struct la_block { static constexpr int tokens = RR == 16 ? 8 : 16; };
+
+template <typename T, int RR, bool CH>
 __global__ __launch_bounds__(256)
 void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int ldq, int ldk, int ldv,
                              const float* __restrict__ decay, const float* __restrict__ head_decay, float q_scale,
                              float* __restrict__ state, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots,
                              float* __restrict__ out, int H, int D, int V, int keep) {
-    extern __shared__ float sm[];                   // [2][3 * D + LA_VC]
+    constexpr int Dp = LA_DG * RR;                  // key channels, padded
+    constexpr int NQ = CH ? 3 : 2;                  // rows of Dp a token: q, k and, per channel, the decay
+    constexpr int per = NQ * Dp + LA_VC;
+    constexpr int U = (per + 255) / 256;
+    constexpr int TB = la_block<RR>::tokens;
+    extern __shared__ __attribute__((aligned(16))) float sm[];      // max(2 * TB * per, Dp * 17) floats
     const int e = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * LA_VC;
     const int tid = threadIdx.x, vc = tid / LA_DG, dg = tid % LA_DG;
     const int t_lo = cu_seqlens[e], t_hi = cu_seqlens[e + 1];
     if (t_lo >= t_hi) return;
-    const int R = (D + LA_DG - 1) / LA_DG;
     const int vcol = v0 + vc;
     const bool vok = vcol < V;
     float* srow = state + ((size_t)seq_slots[e] * H + h) * (size_t)D * V;
-    float S[LA_MAXR];
-#pragma unroll
-    for (int r = 0; r < LA_MAXR; ++r) {
-        const int d = dg + r * LA_DG;
-        S[r] = (r < R && d < D && vok) ? srow[(size_t)d * V + vcol] : 0.f;
+    for (int i = tid; i < D * LA_VC; i += 256) {
+        const int d = i / LA_VC, c = i % LA_VC;
+        sm[d * (LA_VC + 1) + c] = v0 + c < V ? srow[(size_t)d * V + v0 + c] : 0.f;
     }
-    const int per = 3 * D + LA_VC;
-    const float hd = head_decay ? head_decay[h] : 1.f;
-    // what a thread fetches for a token: element i of [q | k | decay | v slice]
+    __syncthreads();
+    float S[RR];
+#pragma unroll
+    for (int r = 0; r < RR; ++r) {
+        const int d = dg * RR + r;
+        S[r] = d < D ? sm[d * (LA_VC + 1) + vc] : 0.f;
+    }
+    __syncthreads();
+    const float hd = CH ? 1.f : head_decay[h];
+    // element i of a token's row in LDS: [q | k | decay | v slice], each of the first padded with zeros
     auto fetch = [&](int t, int i) -> float {
-        if (i < D) return to_f32<T>(q[(size_t)t * ldq + h * D + i]) * q_scale;
-        if (i < 2 * D) return to_f32<T>(k[(size_t)t * ldk + h * D + (i - D)]);
-        if (i < 3 * D) return decay ? decay[((size_t)t * H + h) * D + (i - 2 * D)] : hd;
-        const int c = v0 + (i - 3 * D);
+        const int part = i / Dp, d = i % Dp;
+        if (part < NQ) {
+            if (d >= D) return 0.f;
+            if (part == 0) return to_f32<T>(q[(size_t)t * ldq + h * D + d]) * q_scale;
+            if (part == 1) return to_f32<T>(k[(size_t)t * ldk + h * D + d]);
+            return decay[((size_t)t * H + h) * D + d];
+        }
+        const int c = v0 + (i - NQ * Dp);
         return c < V ? to_f32<T>(v[(size_t)t * ldv + h * V + c]) : 0.f;
     };
-    // up to four elements a thread (3 * 256 + 16 <= 4 * 256)
-    float nx[4];
+    float nx[TB][U];
+    auto load = [&](int t0) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) { const int i = tid + u * 256; nx[u] = i < per ? fetch(t_lo, i) : 0.f; }
+        for (int j = 0; j < TB; ++j)
 #pragma unroll
-    for (int u = 0; u < 4; ++u) { const int i = tid + u * 256; if (i < per) sm[i] = nx[u]; }
-    __syncthreads();
-    for (int t = t_lo; t < t_hi; ++t) {
-        const float* cur = sm + ((t - t_lo) & 1) * per;
-        float* nxt = sm + (((t - t_lo) & 1) ^ 1) * per;
-        if (t + 1 < t_hi) {
-#pragma unroll
-            for (int u = 0; u < 4; ++u) { const int i = tid + u * 256; nx[u] = i < per ? fetch(t + 1, i) : 0.f; }
-        }
-        const float vv = cur[3 * D + vc];
-        float acc = 0.f;
-#pragma unroll
-        for (int r = 0; r < LA_MAXR; ++r) {
-            const int d = dg + r * LA_DG;
-            if (r < R && d < D) {
-                S[r] = fmaf(cur[2 * D + d], S[r], cur[D + d] * vv);
-                acc = fmaf(S[r], cur[d], acc);
+            for (int u = 0; u < U; ++u) {
+                const int i = tid + u * 256;
+                if (t0 + j < t_hi && i < per) nx[j][u] = fetch(t0 + j, i);
             }
-        }
-        acc += __shfl_xor(acc, 1, 64);
-        acc += __shfl_xor(acc, 2, 64);
-        acc += __shfl_xor(acc, 4, 64);
-        acc += __shfl_xor(acc, 8, 64);
-        if (dg == 0 && vok) out[((size_t)t * H + h) * V + vcol] = acc;
-        if (t + 1 < t_hi) {
+    };
+    auto put = [&](float* buf, int t0) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) { const int i = tid + u * 256; if (i < per) nxt[i] = nx[u]; }
+        for (int j = 0; j < TB; ++j)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = tid + u * 256;
+                if (t0 + j < t_hi && i < per) buf[j * per + i] = nx[j][u];
+            }
+    };
+    load(t_lo);
+    put(sm, t_lo);
+    __syncthreads();
+    int b = 0;
+    for (int t0 = t_lo; t0 < t_hi; t0 += TB, b ^= 1) {
+        const float* cur = sm + b * (TB * per);
+        if (t0 + TB < t_hi) load(t0 + TB);
+        const int nb = t_hi - t0 < TB ? t_hi - t0 : TB;
+        for (int j = 0; j < nb; ++j) {
+            const float* row = cur + j * per;
+            const float vv = row[NQ * Dp + vc];
+            float qv[RR], kv[RR], av[RR];
+#pragma unroll
+            for (int r = 0; r < RR; r += 4) {
+                const float4 q4 = *(const float4*)(row + dg * RR + r);
+                const float4 k4 = *(const float4*)(row + Dp + dg * RR + r);
+                qv[r] = q4.x, qv[r + 1] = q4.y, qv[r + 2] = q4.z, qv[r + 3] = q4.w;
+                kv[r] = k4.x, kv[r + 1] = k4.y, kv[r + 2] = k4.z, kv[r + 3] = k4.w;
+                if (CH) {
+                    const float4 a4 = *(const float4*)(row + 2 * Dp + dg * RR + r);
+                    av[r] = a4.x, av[r + 1] = a4.y, av[r + 2] = a4.z, av[r + 3] = a4.w;
+                }
+            }
+            float acc = 0.f;
+#pragma unroll
+            for (int r = 0; r < RR; ++r) {
+                S[r] = fmaf(CH ? av[r] : hd, S[r], kv[r] * vv);
+                acc = fmaf(S[r], qv[r], acc);
+            }
+            acc += __shfl_xor(acc, 1, 64);
+            acc += __shfl_xor(acc, 2, 64);
+            acc += __shfl_xor(acc, 4, 64);
+            acc += __shfl_xor(acc, 8, 64);
+            if (dg == 0 && vok) out[((size_t)(t0 + j) * H + h) * V + vcol] = acc;
         }
+        if (t0 + TB < t_hi) put(sm + (b ^ 1) * (TB * per), t0 + TB);
         __syncthreads();
     }
     if (keep) {
 #pragma unroll
-        for (int r = 0; r < LA_MAXR; ++r) {
-            const int d = dg + r * LA_DG;
-            if (r < R && d < D && vok) srow[(size_t)d * V + vcol] = S[r];
+        for (int r = 0; r < RR; ++r) {
+            const int d = dg * RR + r;
+            if (d < D) sm[d * (LA_VC + 1) + vc] = S[r];
+        }
+        __syncthreads();
+        for (int i = tid; i < D * LA_VC; i += 256) {
+            const int d = i / LA_VC, c = i % LA_VC;
+            if (v0 + c < V) srow[(size_t)d * V + v0 + c] = sm[d * (LA_VC + 1) + c];
         }
     }
+}
+
+template <typename T, int RR, bool CH>
+static void la_launch(dim3 grid, hipStream_t st, const void* q, const void* k, const void* v, int ldq, int ldk, int ldv,
+                      const float* decay, const float* head_decay, float q_scale, float* state, const int* cu_seqlens,
+                      const int* seq_slots, float* out, int H, int D, int V, int keep) {
+    constexpr int Dp = LA_DG * RR, per = (CH ? 3 : 2) * Dp + LA_VC, TB = la_block<RR>::tokens;
+    constexpr size_t a = (size_t)2 * TB * per, b = (size_t)Dp * (LA_VC + 1);
+    static_assert((a > b ? a : b) * sizeof(float) <= 64 * 1024, "linear_attn_scan: the token blocks must fit the default LDS limit");
+    linear_attn_scan_kernel<T, RR, CH><<<grid, 256, (a > b ? a : b) * sizeof(float), st>>>(
+        (const T*)q, (const T*)k, (const T*)v, ldq, ldk, ldv, decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, D, V, keep);
+}
+
+template <typename T>
+static void la_pick(int D, bool ch, dim3 grid, hipStream_t st, const void* q, const void* k, const void* v, int ldq, int ldk, int ldv,
+                    const float* decay, const float* head_decay, float q_scale, float* state, const int* cu_seqlens,
+                    const int* seq_slots, float* out, int H, int V, int keep) {
+#define LA_GO(RR, CH) la_launch<T, RR, CH>(grid, st, q, k, v, ldq, ldk, ldv, decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, D, V, keep)
+    if (D <= 64) { if (ch) LA_GO(4, true); else LA_GO(4, false); }
+    else if (D <= 128) { if (ch) LA_GO(8, true); else LA_GO(8, false); }
+    else { if (ch) LA_GO(16, true); else LA_GO(16, false); }
+#undef LA_GO
 }
 
 extern "C" int spite_linear_attn_scan(const void* q, const void* k, const void* v, int ldq, int ldk, int ldv, int dtype,
@@ -127,19 +194,16 @@ extern "C" int spite_linear_attn_scan(const void* q, const void* k, const void* 
                                       const int* cu_seqlens, const int* seq_slots, int n_seqs, float* out,
                                       int H, int D, int V, int keep, hipStream_t st) {
     SP_REQUIRE(n_seqs >= 0 && H > 0 && D > 0 && V > 0 && n_slots > 0, "linear_attn_scan: bad sizes");
-    SP_REQUIRE(D <= LA_DG * LA_MAXR, "linear_attn_scan: %d key channels a head (at most %d)", D, LA_DG * LA_MAXR);
+    SP_REQUIRE(D <= LA_MAXD, "linear_attn_scan: %d key channels a head (at most %d)", D, LA_MAXD);
     SP_REQUIRE(ldq >= H * D && ldk >= H * D && ldv >= H * V, "linear_attn_scan: rows shorter than the heads");
     SP_REQUIRE((decay != nullptr) != (head_decay != nullptr), "linear_attn_scan: a decay per channel or one per head, one of them");
     SP_REQUIRE(H <= 65535 && (V + LA_VC - 1) / LA_VC <= 65535, "linear_attn_scan: too many heads or value columns");
     if (n_seqs == 0) return 0;
     const dim3 grid(n_seqs, H, (V + LA_VC - 1) / LA_VC);
-    const size_t sh = (size_t)2 * (3 * D + LA_VC) * sizeof(float);
     if (dtype == SP_F32)
-        linear_attn_scan_kernel<float><<<grid, 256, sh, st>>>((const float*)q, (const float*)k, (const float*)v, ldq, ldk, ldv,
-            decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, D, V, keep);
+        la_pick<float>(D, decay != nullptr, grid, st, q, k, v, ldq, ldk, ldv, decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, V, keep);
     else if (dtype == SP_BF16)
-        linear_attn_scan_kernel<bf16><<<grid, 256, sh, st>>>((const bf16*)q, (const bf16*)k, (const bf16*)v, ldq, ldk, ldv,
-            decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, D, V, keep);
+        la_pick<bf16>(D, decay != nullptr, grid, st, q, k, v, ldq, ldk, ldv, decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, V, keep);
     else return sp_fail("linear_attn_scan: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("linear_attn_scan");
     return 0;

@@ -157,6 +157,14 @@ def random_tensors(config: dict, seed: int, std: float = 0.02, device=None) -> D
     return out
 
 
+def free_axes(config: dict) -> Dict[str, tuple]:
+    """{checkpoint name: axes whose size the checkpoint decides} for the tensors of ``config`` that have any."""
+    from ..engine.model import Model
+    arch, cfg = read_config(config)
+    model = Model(arch.build_spec(cfg), Env(torch.float32, torch.device("cpu")))
+    return {fname: tuple(ps.free) for fname, ps, _, _ in model.tensor_plan() if ps.free}
+
+
 def write_random_model(folder: str, config: dict, seed: int, std: float = 0.02, dtype: str | None = None,
                        overrides: Dict[str, torch.Tensor] | None = None, device=None, keep_wide=()) -> str:
     """Writes ``folder/config.json`` and ``folder/model.safetensors``; returns the folder.
@@ -171,11 +179,14 @@ def write_random_model(folder: str, config: dict, seed: int, std: float = 0.02, 
         raise ValueError(f"dtype {dtype!r} (known: {sorted(_FILE_DTYPES)})")
     config["torch_dtype"] = dtype
     tensors = random_tensors(config, seed, std, device)
+    free = free_axes(config) if overrides else {}
     for name, t in (overrides or {}).items():
         if name not in tensors:
             raise KeyError(f"override for unknown tensor {name!r}")
-        if tuple(t.shape) != tuple(tensors[name].shape):
-            raise ValueError(f"override for {name}: shape {tuple(t.shape)}, expected {tuple(tensors[name].shape)}")
+        want = tuple(tensors[name].shape)
+        # (a size that the checkpoint decides may differ from what random weights are drawn with)
+        if len(t.shape) != len(want) or any(a != e and ax not in free.get(name, ()) for ax, (a, e) in enumerate(zip(t.shape, want))):
+            raise ValueError(f"override for {name}: shape {tuple(t.shape)}, expected {want}")
         tensors[name] = t.to(torch.float32) if t.is_floating_point() else t
     wide = lambda n: any(k in n for k in keep_wide)
     stored = {n: (t.to(torch.float32 if wide(n) else _FILE_DTYPES[dtype]) if t.is_floating_point() else t)
