@@ -52,7 +52,20 @@ extern "C" int spite_channel_decay(float* z, const float* bias, int T, int width
 
 template <int RR> struct la_block { static constexpr int tokens = RR == 16 ? 8 : 16; };
 
-template <typename T, int RR, bool CH>
+// The sum over the 16 lanes of a row, by rotations within the row (no LDS traffic); every lane gets it.
+__device__ __forceinline__ float row16_sum(float x) {
+#define LA_ROR(n) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 | (n), 0xf, 0xf, false))
+    x += LA_ROR(8);
+    x += LA_ROR(4);
+    x += LA_ROR(2);
+    x += LA_ROR(1);
+#undef LA_ROR
+    return x;
+}
+
+// VEC: q, k, v (bfloat16) and the decay rows start on 16 bytes and D and V are multiples of 8: a thread
+// fetches eight elements at a time.  Otherwise one element at a time.
+template <typename T, int RR, bool CH, bool VEC>
 __global__ __launch_bounds__(256)
 void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int ldq, int ldk, int ldv,
                              const float* __restrict__ decay, const float* __restrict__ head_decay, float q_scale,
@@ -61,8 +74,10 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
     constexpr int Dp = LA_DG * RR;                  // key channels, padded
     constexpr int NQ = CH ? 3 : 2;                  // rows of Dp a token: q, k and, per channel, the decay
     constexpr int per = NQ * Dp + LA_VC;
-    constexpr int U = (per + 255) / 256;
     constexpr int TB = la_block<RR>::tokens;
+    constexpr int W = VEC ? 8 : 1;                  // elements a fetch
+    constexpr int CPT = per / W;                    // fetches a token
+    constexpr int U = (TB * CPT + 255) / 256;       // fetches a thread and block
     extern __shared__ __attribute__((aligned(16))) float sm[];      // max(2 * TB * per, Dp * 17) floats
     const int e = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * LA_VC;
     const int tid = threadIdx.x, vc = tid / LA_DG, dg = tid % LA_DG;
@@ -84,36 +99,71 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
     }
     __syncthreads();
     const float hd = CH ? 1.f : head_decay[h];
-    // element i of a token's row in LDS: [q | k | decay | v slice], each of the first padded with zeros
-    auto fetch = [&](int t, int i) -> float {
-        const int part = i / Dp, d = i % Dp;
-        if (part < NQ) {
-            if (d >= D) return 0.f;
-            if (part == 0) return to_f32<T>(q[(size_t)t * ldq + h * D + d]) * q_scale;
-            if (part == 1) return to_f32<T>(k[(size_t)t * ldk + h * D + d]);
-            return decay[((size_t)t * H + h) * D + d];
+    // elements [W i, W i + W) of a token's row in LDS: [q | k | decay | v slice], each of the first padded with zeros
+    auto fetch = [&](int t, int i, float* dst) {
+        const int part = (i * W) / Dp, d = (i * W) % Dp;
+        if constexpr (VEC) {
+#pragma unroll
+            for (int x = 0; x < 8; ++x) dst[x] = 0.f;
+            if (part < NQ) {
+                if (d >= D) return;
+                if (part == 2) {
+                    const float4* src = (const float4*)(decay + ((size_t)t * H + h) * D + d);
+                    const float4 a = src[0], b = src[1];
+                    dst[0] = a.x, dst[1] = a.y, dst[2] = a.z, dst[3] = a.w, dst[4] = b.x, dst[5] = b.y, dst[6] = b.z, dst[7] = b.w;
+                    return;
+                }
+                const uint4 raw = *(const uint4*)(part == 0 ? (const void*)(q + (size_t)t * ldq + h * D + d) : (const void*)(k + (size_t)t * ldk + h * D + d));
+                const unsigned wds[4] = {raw.x, raw.y, raw.z, raw.w};
+                const float m = part == 0 ? q_scale : 1.f;
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    dst[2 * x] = __builtin_bit_cast(float, wds[x] << 16) * m;
+                    dst[2 * x + 1] = __builtin_bit_cast(float, wds[x] & 0xffff0000u) * m;
+                }
+                return;
+            }
+            const int c = v0 + (i * W - NQ * Dp);
+            if (c >= V) return;
+            const uint4 raw = *(const uint4*)(v + (size_t)t * ldv + h * V + c);
+            const unsigned wds[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                dst[2 * x] = __builtin_bit_cast(float, wds[x] << 16);
+                dst[2 * x + 1] = __builtin_bit_cast(float, wds[x] & 0xffff0000u);
+            }
+        } else {
+            if (part < NQ) {
+                if (d >= D) dst[0] = 0.f;
+                else if (part == 0) dst[0] = to_f32<T>(q[(size_t)t * ldq + h * D + d]) * q_scale;
+                else if (part == 1) dst[0] = to_f32<T>(k[(size_t)t * ldk + h * D + d]);
+                else dst[0] = decay[((size_t)t * H + h) * D + d];
+                return;
+            }
+            const int c = v0 + (i - NQ * Dp);
+            dst[0] = c < V ? to_f32<T>(v[(size_t)t * ldv + h * V + c]) : 0.f;
         }
-        const int c = v0 + (i - NQ * Dp);
-        return c < V ? to_f32<T>(v[(size_t)t * ldv + h * V + c]) : 0.f;
     };
-    float nx[TB][U];
+    float nx[U][W];
     auto load = [&](int t0) {
 #pragma unroll
-        for (int j = 0; j < TB; ++j)
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int i = tid + u * 256;
-                if (t0 + j < t_hi && i < per) nx[j][u] = fetch(t0 + j, i);
-            }
+        for (int u = 0; u < U; ++u) {
+            const int x = tid + u * 256, j = x / CPT, i = x % CPT;
+            if (j < TB && t0 + j < t_hi) fetch(t0 + j, i, nx[u]);
+        }
     };
     auto put = [&](float* buf, int t0) {
 #pragma unroll
-        for (int j = 0; j < TB; ++j)
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int i = tid + u * 256;
-                if (t0 + j < t_hi && i < per) buf[j * per + i] = nx[j][u];
+        for (int u = 0; u < U; ++u) {
+            const int x = tid + u * 256, j = x / CPT, i = x % CPT;
+            if (j < TB && t0 + j < t_hi) {
+                float* dst = buf + j * per + i * W;
+                if constexpr (VEC) {
+                    *(float4*)dst = make_float4(nx[u][0], nx[u][1], nx[u][2], nx[u][3]);
+                    *(float4*)(dst + 4) = make_float4(nx[u][4], nx[u][5], nx[u][6], nx[u][7]);
+                } else dst[0] = nx[u][0];
             }
+        }
     };
     load(t_lo);
     put(sm, t_lo);
@@ -123,7 +173,9 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
         const float* cur = sm + b * (TB * per);
         if (t0 + TB < t_hi) load(t0 + TB);
         const int nb = t_hi - t0 < TB ? t_hi - t0 : TB;
-        for (int j = 0; j < nb; ++j) {
+        float* orow = out + ((size_t)t0 * H + h) * V + vcol;
+        // one token: the state moves on, and the thread's part of the sum over the key channels comes back
+        auto token = [&](int j) -> float {
             const float* row = cur + j * per;
             const float vv = row[NQ * Dp + vc];
             float qv[RR], kv[RR], av[RR];
@@ -144,11 +196,25 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
                 S[r] = fmaf(CH ? av[r] : hd, S[r], kv[r] * vv);
                 acc = fmaf(S[r], qv[r], acc);
             }
-            acc += __shfl_xor(acc, 1, 64);
-            acc += __shfl_xor(acc, 2, 64);
-            acc += __shfl_xor(acc, 4, 64);
-            acc += __shfl_xor(acc, 8, 64);
-            if (dg == 0 && vok) out[((size_t)(t0 + j) * H + h) * V + vcol] = acc;
+            return acc;
+        };
+        if (nb == TB) {
+            // a whole block as one stretch of code: only the state's FMA waits for the token before, the reads,
+            // the sums across lanes and the stores of different tokens overlap
+            float accs[TB];
+#pragma unroll
+            for (int j = 0; j < TB; ++j) accs[j] = token(j);
+#pragma unroll
+            for (int j = 0; j < TB; ++j) accs[j] = row16_sum(accs[j]);
+            if (dg == 0 && vok) {
+#pragma unroll
+                for (int j = 0; j < TB; ++j) orow[(size_t)j * H * V] = accs[j];
+            }
+        } else {
+            for (int j = 0; j < nb; ++j) {
+                const float acc = row16_sum(token(j));
+                if (dg == 0 && vok) orow[(size_t)j * H * V] = acc;
+            }
         }
         if (t0 + TB < t_hi) put(sm + (b ^ 1) * (TB * per), t0 + TB);
         __syncthreads();
@@ -167,26 +233,28 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
     }
 }
 
-template <typename T, int RR, bool CH>
-static void la_launch(dim3 grid, hipStream_t st, const void* q, const void* k, const void* v, int ldq, int ldk, int ldv,
-                      const float* decay, const float* head_decay, float q_scale, float* state, const int* cu_seqlens,
-                      const int* seq_slots, float* out, int H, int D, int V, int keep) {
+struct la_args {
+    dim3 grid; hipStream_t st; const void *q, *k, *v; int ldq, ldk, ldv; const float *decay, *head_decay; float q_scale;
+    float* state; const int *cu_seqlens, *seq_slots; float* out; int H, D, V, keep;
+};
+
+template <typename T, int RR, bool CH, bool VEC>
+static void la_launch(const la_args& a) {
     constexpr int Dp = LA_DG * RR, per = (CH ? 3 : 2) * Dp + LA_VC, TB = la_block<RR>::tokens;
-    constexpr size_t a = (size_t)2 * TB * per, b = (size_t)Dp * (LA_VC + 1);
-    static_assert((a > b ? a : b) * sizeof(float) <= 64 * 1024, "linear_attn_scan: the token blocks must fit the default LDS limit");
-    linear_attn_scan_kernel<T, RR, CH><<<grid, 256, (a > b ? a : b) * sizeof(float), st>>>(
-        (const T*)q, (const T*)k, (const T*)v, ldq, ldk, ldv, decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, D, V, keep);
+    constexpr size_t blocks = (size_t)2 * TB * per, tile = (size_t)Dp * (LA_VC + 1);
+    constexpr size_t bytes = (blocks > tile ? blocks : tile) * sizeof(float);
+    static_assert(bytes <= 64 * 1024, "linear_attn_scan: the token blocks must fit the default LDS limit");
+    linear_attn_scan_kernel<T, RR, CH, VEC><<<a.grid, 256, bytes, a.st>>>(
+        (const T*)a.q, (const T*)a.k, (const T*)a.v, a.ldq, a.ldk, a.ldv, a.decay, a.head_decay, a.q_scale, a.state, a.cu_seqlens,
+        a.seq_slots, a.out, a.H, a.D, a.V, a.keep);
 }
 
-template <typename T>
-static void la_pick(int D, bool ch, dim3 grid, hipStream_t st, const void* q, const void* k, const void* v, int ldq, int ldk, int ldv,
-                    const float* decay, const float* head_decay, float q_scale, float* state, const int* cu_seqlens,
-                    const int* seq_slots, float* out, int H, int V, int keep) {
-#define LA_GO(RR, CH) la_launch<T, RR, CH>(grid, st, q, k, v, ldq, ldk, ldv, decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, D, V, keep)
-    if (D <= 64) { if (ch) LA_GO(4, true); else LA_GO(4, false); }
-    else if (D <= 128) { if (ch) LA_GO(8, true); else LA_GO(8, false); }
-    else { if (ch) LA_GO(16, true); else LA_GO(16, false); }
-#undef LA_GO
+template <typename T, bool VEC>
+static void la_pick(const la_args& a) {
+    const bool ch = a.decay != nullptr;
+    if (a.D <= 64) { if (ch) la_launch<T, 4, true, VEC>(a); else la_launch<T, 4, false, VEC>(a); }
+    else if (a.D <= 128) { if (ch) la_launch<T, 8, true, VEC>(a); else la_launch<T, 8, false, VEC>(a); }
+    else { if (ch) la_launch<T, 16, true, VEC>(a); else la_launch<T, 16, false, VEC>(a); }
 }
 
 extern "C" int spite_linear_attn_scan(const void* q, const void* k, const void* v, int ldq, int ldk, int ldv, int dtype,
@@ -198,13 +266,16 @@ extern "C" int spite_linear_attn_scan(const void* q, const void* k, const void* 
     SP_REQUIRE(ldq >= H * D && ldk >= H * D && ldv >= H * V, "linear_attn_scan: rows shorter than the heads");
     SP_REQUIRE((decay != nullptr) != (head_decay != nullptr), "linear_attn_scan: a decay per channel or one per head, one of them");
     SP_REQUIRE(H <= 65535 && (V + LA_VC - 1) / LA_VC <= 65535, "linear_attn_scan: too many heads or value columns");
+    SP_REQUIRE(dtype == SP_F32 || dtype == SP_BF16, "linear_attn_scan: unknown dtype %d", dtype);
     if (n_seqs == 0) return 0;
-    const dim3 grid(n_seqs, H, (V + LA_VC - 1) / LA_VC);
-    if (dtype == SP_F32)
-        la_pick<float>(D, decay != nullptr, grid, st, q, k, v, ldq, ldk, ldv, decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, V, keep);
-    else if (dtype == SP_BF16)
-        la_pick<bf16>(D, decay != nullptr, grid, st, q, k, v, ldq, ldk, ldv, decay, head_decay, q_scale, state, cu_seqlens, seq_slots, out, H, V, keep);
-    else return sp_fail("linear_attn_scan: unknown dtype %d", dtype);
+    const la_args a{dim3(n_seqs, H, (V + LA_VC - 1) / LA_VC), st, q, k, v, ldq, ldk, ldv, decay, head_decay, q_scale, state,
+                    cu_seqlens, seq_slots, out, H, D, V, keep};
+    auto on16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    const bool vec = dtype == SP_BF16 && D % 8 == 0 && V % 8 == 0 && ldq % 8 == 0 && ldk % 8 == 0 && ldv % 8 == 0
+                     && on16(q) && on16(k) && on16(v) && on16(decay);
+    if (dtype == SP_F32) la_pick<float, false>(a);
+    else if (vec) la_pick<bf16, true>(a);
+    else la_pick<bf16, false>(a);
     SP_LAUNCH_CHECK("linear_attn_scan");
     return 0;
 }

@@ -280,7 +280,7 @@ def test_plain_mechanisms():
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("kind", ["channel", "head"])
 @pytest.mark.parametrize("Hh,D,V,lens", [(3, 6, 10, [5, 1, 2, 1]), (2, 64, 64, [150, 1, 67]), (1, 130, 20, [33]), (2, 32, 128, [64, 128]),
-                                         (4, 128, 128, [1, 1, 1, 1])])
+                                         (4, 128, 128, [1, 1, 1, 1]), (1, 256, 72, [40, 3])])
 def test_linear_attention_kernel(dtype, kind, Hh, D, V, lens):
     """Portions and single tokens of several requests in two steps through state rows that lie apart: the
     second step goes on from what the first left, nobody reads or writes another slot's row."""
