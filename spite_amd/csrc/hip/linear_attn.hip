@@ -13,6 +13,7 @@
 // gated_group_norm:   y = rmsnorm(o over groups of `group` elements) * w * act(gate), the step between the
 //                     recurrence and the output projection.
 #include "common.h"
+#include <type_traits>
 
 // ------------------------------------------------------------------ decay per channel
 // a = sigmoid(z + b)^(1/tau) = exp(log sigmoid(z + b) / tau), log sigmoid(x) = -(max(-x, 0) + log1p(exp(-|x|))).
@@ -37,16 +38,19 @@ extern "C" int spite_channel_decay(float* z, const float* bias, int T, int width
 }
 
 // ------------------------------------------------------------------ the recurrence, token by token
-// A workgroup of 256 threads takes 16 value columns of one head of one entry of the step and walks the
-// entry's tokens in order.  Thread (vc, dg) = (tid / 16, tid % 16) holds the state's elements
-// S[dg * RR + r][v0 + vc], r < RR (RR = 4, 8 or 16 for up to 64, 128 or 256 key channels), in registers.
-// The tokens' q, k, decay and value slice go through LDS a block of LA_TB tokens at a time, two buffers:
-// the next block's loads are in flight while this block is computed, so a token costs its FMAs, a few
-// wide LDS reads and four steps across the thread's 16 neighbours, and one barrier a block.  The
-// dependent chain from token to token is the one FMA of the state.  The state tile goes through LDS on
+// A workgroup of 128 threads takes 16 value columns of one head of one entry of the step and walks the
+// entry's tokens in order.  Thread (vc, dg) = (tid / 16, tid % 16) holds, in registers, the state's elements
+// S[d][v0 + vc] and S[d][v0 + vc + 8] for the key channels d = 64 m + 4 dg + x (x < 4, m < RR / 4; RR = 4, 8 or
+// 16 for up to 64, 128 or 256 key channels): 16 lanes read 256 consecutive bytes of a token's q, k or decay
+// row from LDS in one wide read without bank conflicts, and every such read serves two columns (LDS reads,
+// not FMAs, bound the walk).  The tokens' q, k, decay and value slice go through LDS a block of tokens at a
+// time, two buffers: the next block's loads are in flight while this block is computed, and a whole block is
+// one stretch of code: only the state's FMA waits for the token before.  The sum over the key channels is a
+// thread's own partial sum and four rotations across its 16 neighbours.  The state tile goes through LDS on
 // the way in and out, so that its rows are read and written 64 bytes at a time.
 // The order of every sum is fixed by D alone: the bits do not depend on how a request's tokens are cut.
-#define LA_VC 16
+#define LA_VC 16        // value columns a workgroup
+#define LA_NT 128       // threads a workgroup: 8 x 16, two columns a thread
 #define LA_DG 16
 #define LA_MAXD 256
 
@@ -63,10 +67,13 @@ __device__ __forceinline__ float row16_sum(float x) {
     return x;
 }
 
-// VEC: q, k, v (bfloat16) and the decay rows start on 16 bytes and D and V are multiples of 8: a thread
-// fetches eight elements at a time.  Otherwise one element at a time.
-template <typename T, int RR, bool CH, bool VEC>
-__global__ __launch_bounds__(256)
+// VEC: q, k, v (bfloat16) and the decay rows start on 16 bytes and D and V are multiples of 8: a fetch is
+// 16 bytes.  Otherwise one element.  (Plain loops and no closures: every array below stays in registers.)
+#define LA_OWN(r) (((r) / 4) * 64 + dg * 4 + ((r) % 4))          // the thread's r-th key channel
+// TB: tokens a block: 16 (8 for the widest heads), or 1 for steps of single tokens, whose workgroups then hold
+// little LDS and few registers, so that many are resident and their round trips to memory overlap.
+template <typename T, int RR, bool CH, bool VEC, int TB>
+__global__ __launch_bounds__(LA_NT) __attribute__((amdgpu_waves_per_eu(1, TB == 1 ? 4 : 2)))
 void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, int ldq, int ldk, int ldv,
                              const float* __restrict__ decay, const float* __restrict__ head_decay, float q_scale,
                              float* __restrict__ state, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots,
@@ -74,193 +81,198 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
     constexpr int Dp = LA_DG * RR;                  // key channels, padded
     constexpr int NQ = CH ? 3 : 2;                  // rows of Dp a token: q, k and, per channel, the decay
     constexpr int per = NQ * Dp + LA_VC;
-    constexpr int TB = la_block<RR>::tokens;
-    constexpr int W = VEC ? 8 : 1;                  // elements a fetch
-    constexpr int CPT = per / W;                    // fetches a token
-    constexpr int U = (TB * CPT + 255) / 256;       // fetches a thread and block
+    // A fetch is one load and no branch around it.  Two lists of fetches a block: A from q, k and the value
+    // slice (elements of type T), B from the decay rows (fp32).
+    constexpr int WA = VEC ? 8 : 1, WB = VEC ? 4 : 1;               // elements a fetch
+    constexpr int CA = (2 * Dp + LA_VC) / WA, CB = CH ? Dp / WB : 1; // fetches a token
+    constexpr int UA = (TB * CA + LA_NT - 1) / LA_NT, UB = CH ? (TB * CB + LA_NT - 1) / LA_NT : 0;   // fetches a thread and block
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    using RawA = typename std::conditional<VEC, u32x4, T>::type;
+    using RawB = typename std::conditional<VEC, f32x4, float>::type;
     extern __shared__ __attribute__((aligned(16))) float sm[];      // max(2 * TB * per, Dp * 17) floats
     const int e = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * LA_VC;
     const int tid = threadIdx.x, vc = tid / LA_DG, dg = tid % LA_DG;
     const int t_lo = cu_seqlens[e], t_hi = cu_seqlens[e + 1];
     if (t_lo >= t_hi) return;
-    const int vcol = v0 + vc;
-    const bool vok = vcol < V;
+    const int vcol = v0 + vc;                       // and vcol + 8
+    const bool vok = vcol < V, vok2 = vcol + 8 < V;
     float* srow = state + ((size_t)seq_slots[e] * H + h) * (size_t)D * V;
-    for (int i = tid; i < D * LA_VC; i += 256) {
+    for (int i = tid; i < D * LA_VC; i += LA_NT) {
         const int d = i / LA_VC, c = i % LA_VC;
         sm[d * (LA_VC + 1) + c] = v0 + c < V ? srow[(size_t)d * V + v0 + c] : 0.f;
     }
     __syncthreads();
-    float S[RR];
+    float S[RR], S2[RR];
 #pragma unroll
     for (int r = 0; r < RR; ++r) {
-        const int d = dg * RR + r;
+        const int d = LA_OWN(r);
         S[r] = d < D ? sm[d * (LA_VC + 1) + vc] : 0.f;
+        S2[r] = d < D ? sm[d * (LA_VC + 1) + vc + 8] : 0.f;
     }
     __syncthreads();
     const float hd = CH ? 1.f : head_decay[h];
-    // elements [W i, W i + W) of a token's row in LDS: [q | k | decay | v slice], each of the first padded with zeros
-    auto fetch = [&](int t, int i, float* dst) {
-        const int part = (i * W) / Dp, d = (i * W) % Dp;
-        if constexpr (VEC) {
+    RawA na[UA];
+    RawB nb[UB > 0 ? UB : 1];
+    // Turn `it` computes block `it` from buffer it & 1 while block it + 1 is on its way into the other one;
+    // turn -1 only fetches.
+    const int n_blocks = (t_hi - t_lo + TB - 1) / TB;
+    for (int it = -1; it < n_blocks; ++it) {
+        const int t0 = t_lo + it * TB, tn = t0 + TB;                // this block's first token, the next block's
+        const bool more = it + 1 < n_blocks;
+        if (more) {
 #pragma unroll
-            for (int x = 0; x < 8; ++x) dst[x] = 0.f;
-            if (part < NQ) {
-                if (d >= D) return;
-                if (part == 2) {
-                    const float4* src = (const float4*)(decay + ((size_t)t * H + h) * D + d);
-                    const float4 a = src[0], b = src[1];
-                    dst[0] = a.x, dst[1] = a.y, dst[2] = a.z, dst[3] = a.w, dst[4] = b.x, dst[5] = b.y, dst[6] = b.z, dst[7] = b.w;
-                    return;
-                }
-                const uint4 raw = *(const uint4*)(part == 0 ? (const void*)(q + (size_t)t * ldq + h * D + d) : (const void*)(k + (size_t)t * ldk + h * D + d));
-                const unsigned wds[4] = {raw.x, raw.y, raw.z, raw.w};
-                const float m = part == 0 ? q_scale : 1.f;
-#pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    dst[2 * x] = __builtin_bit_cast(float, wds[x] << 16) * m;
-                    dst[2 * x + 1] = __builtin_bit_cast(float, wds[x] & 0xffff0000u) * m;
-                }
-                return;
+            for (int u = 0; u < UA; ++u) {
+                const int x = tid + u * LA_NT, j = x / CA, e0 = (x % CA) * WA, part = e0 / Dp, d = e0 % Dp;
+                // q and k: channel d of the head; the value slice: column v0 + e0 - 2 Dp
+                const T* base = part == 0 ? q : part == 1 ? k : v;
+                const int ld = part == 0 ? ldq : part == 1 ? ldk : ldv;
+                const int col = part < 2 ? h * D + d : h * V + v0 + (e0 - 2 * Dp);
+                const bool ok = j < TB && tn + j < t_hi && (part < 2 ? d < D : v0 + (e0 - 2 * Dp) < V);
+                const RawA got = *(const RawA*)(base + (size_t)(ok ? tn + j : t_lo) * ld + (ok ? col : 0));
+                na[u] = ok ? got : RawA{};
             }
-            const int c = v0 + (i * W - NQ * Dp);
-            if (c >= V) return;
-            const uint4 raw = *(const uint4*)(v + (size_t)t * ldv + h * V + c);
-            const unsigned wds[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-            for (int x = 0; x < 4; ++x) {
-                dst[2 * x] = __builtin_bit_cast(float, wds[x] << 16);
-                dst[2 * x + 1] = __builtin_bit_cast(float, wds[x] & 0xffff0000u);
-            }
-        } else {
-            if (part < NQ) {
-                if (d >= D) dst[0] = 0.f;
-                else if (part == 0) dst[0] = to_f32<T>(q[(size_t)t * ldq + h * D + d]) * q_scale;
-                else if (part == 1) dst[0] = to_f32<T>(k[(size_t)t * ldk + h * D + d]);
-                else dst[0] = decay[((size_t)t * H + h) * D + d];
-                return;
-            }
-            const int c = v0 + (i - NQ * Dp);
-            dst[0] = c < V ? to_f32<T>(v[(size_t)t * ldv + h * V + c]) : 0.f;
-        }
-    };
-    float nx[U][W];
-    auto load = [&](int t0) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int x = tid + u * 256, j = x / CPT, i = x % CPT;
-            if (j < TB && t0 + j < t_hi) fetch(t0 + j, i, nx[u]);
-        }
-    };
-    auto put = [&](float* buf, int t0) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int x = tid + u * 256, j = x / CPT, i = x % CPT;
-            if (j < TB && t0 + j < t_hi) {
-                float* dst = buf + j * per + i * W;
-                if constexpr (VEC) {
-                    *(float4*)dst = make_float4(nx[u][0], nx[u][1], nx[u][2], nx[u][3]);
-                    *(float4*)(dst + 4) = make_float4(nx[u][4], nx[u][5], nx[u][6], nx[u][7]);
-                } else dst[0] = nx[u][0];
+            for (int u = 0; u < UB; ++u) {
+                const int x = tid + u * LA_NT, j = x / CB, d = (x % CB) * WB;
+                const bool ok = j < TB && tn + j < t_hi && d < D;
+                const RawB got = *(const RawB*)(decay + ((size_t)(ok ? tn + j : t_lo) * H + h) * D + (ok ? d : 0));
+                nb[u] = ok ? got : RawB{};
             }
         }
-    };
-    load(t_lo);
-    put(sm, t_lo);
-    __syncthreads();
-    int b = 0;
-    for (int t0 = t_lo; t0 < t_hi; t0 += TB, b ^= 1) {
-        const float* cur = sm + b * (TB * per);
-        if (t0 + TB < t_hi) load(t0 + TB);
-        const int nb = t_hi - t0 < TB ? t_hi - t0 : TB;
-        float* orow = out + ((size_t)t0 * H + h) * V + vcol;
-        // one token: the state moves on, and the thread's part of the sum over the key channels comes back
-        auto token = [&](int j) -> float {
-            const float* row = cur + j * per;
-            const float vv = row[NQ * Dp + vc];
-            float qv[RR], kv[RR], av[RR];
-#pragma unroll
-            for (int r = 0; r < RR; r += 4) {
-                const float4 q4 = *(const float4*)(row + dg * RR + r);
-                const float4 k4 = *(const float4*)(row + Dp + dg * RR + r);
-                qv[r] = q4.x, qv[r + 1] = q4.y, qv[r + 2] = q4.z, qv[r + 3] = q4.w;
-                kv[r] = k4.x, kv[r + 1] = k4.y, kv[r + 2] = k4.z, kv[r + 3] = k4.w;
-                if (CH) {
-                    const float4 a4 = *(const float4*)(row + 2 * Dp + dg * RR + r);
-                    av[r] = a4.x, av[r + 1] = a4.y, av[r + 2] = a4.z, av[r + 3] = a4.w;
-                }
-            }
-            float acc = 0.f;
-#pragma unroll
-            for (int r = 0; r < RR; ++r) {
-                S[r] = fmaf(CH ? av[r] : hd, S[r], kv[r] * vv);
-                acc = fmaf(S[r], qv[r], acc);
-            }
-            return acc;
-        };
-        if (nb == TB) {
-            // a whole block as one stretch of code: only the state's FMA waits for the token before, the reads,
+        float accs[TB], accs2[TB];
+        if (it >= 0) {
+            const float* cur = sm + (it & 1) * (TB * per);
+            const int n_tok = t_hi - t0 < TB ? t_hi - t0 : TB;
+            // a whole block as one stretch of code: only the state's FMA waits for the token before; the reads,
             // the sums across lanes and the stores of different tokens overlap
-            float accs[TB];
-#pragma unroll
-            for (int j = 0; j < TB; ++j) accs[j] = token(j);
-#pragma unroll
-            for (int j = 0; j < TB; ++j) accs[j] = row16_sum(accs[j]);
-            if (dg == 0 && vok) {
-#pragma unroll
-                for (int j = 0; j < TB; ++j) orow[(size_t)j * H * V] = accs[j];
+// token j of the block: the state moves on, and the thread's parts of the two sums over the key channels are kept
+#define LA_TOKEN(j)                                                                         \
+            {                                                                               \
+                const float* row = cur + (j) * per;                                         \
+                const float vv = row[NQ * Dp + vc], vv2 = row[NQ * Dp + vc + 8];            \
+                accs[j] = accs2[j] = 0.f;                                                   \
+                _Pragma("unroll")                                                           \
+                for (int r = 0; r < RR; r += 4) {                                           \
+                    const f32x4 q4 = *(const f32x4*)(row + LA_OWN(r));                      \
+                    const f32x4 k4 = *(const f32x4*)(row + Dp + LA_OWN(r));                 \
+                    f32x4 a4 = {hd, hd, hd, hd};                                            \
+                    if (CH) a4 = *(const f32x4*)(row + 2 * Dp + LA_OWN(r));                 \
+                    _Pragma("unroll")                                                       \
+                    for (int y = 0; y < 4; ++y) {                                           \
+                        S[r + y] = fmaf(a4[y], S[r + y], k4[y] * vv);                       \
+                        S2[r + y] = fmaf(a4[y], S2[r + y], k4[y] * vv2);                    \
+                        accs[j] = fmaf(S[r + y], q4[y], accs[j]);                           \
+                        accs2[j] = fmaf(S2[r + y], q4[y], accs2[j]);                        \
+                    }                                                                       \
+                }                                                                           \
             }
-        } else {
-            for (int j = 0; j < nb; ++j) {
-                const float acc = row16_sum(token(j));
-                if (dg == 0 && vok) orow[(size_t)j * H * V] = acc;
+            if (n_tok == TB) {
+                // no branch between the tokens of a whole block
+#pragma unroll
+                for (int j = 0; j < TB; ++j) LA_TOKEN(j)
+            } else {
+#pragma unroll
+                for (int j = 0; j < TB; ++j) {
+                    accs[j] = accs2[j] = 0.f;
+                    if (j < n_tok) LA_TOKEN(j)
+                }
+            }
+#undef LA_TOKEN
+#pragma unroll
+            for (int j = 0; j < TB; ++j) accs[j] = row16_sum(accs[j]), accs2[j] = row16_sum(accs2[j]);
+        }
+        if (more) {
+            float* buf = sm + ((it + 1) & 1) * (TB * per);
+#pragma unroll
+            for (int u = 0; u < UA; ++u) {
+                const int x = tid + u * LA_NT, j = x / CA, e0 = (x % CA) * WA, part = e0 / Dp;
+                if (j < TB && tn + j < t_hi) {
+                    float* dst = buf + j * per + (part < 2 ? e0 : e0 + (NQ - 2) * Dp);
+                    const float m = part == 0 ? q_scale : 1.f;
+                    if constexpr (VEC) {
+                        const u32x4 w = na[u];
+                        f32x4 lo, hi;
+                        lo.x = __builtin_bit_cast(float, w.x << 16) * m, lo.y = __builtin_bit_cast(float, w.x & 0xffff0000u) * m;
+                        lo.z = __builtin_bit_cast(float, w.y << 16) * m, lo.w = __builtin_bit_cast(float, w.y & 0xffff0000u) * m;
+                        hi.x = __builtin_bit_cast(float, w.z << 16) * m, hi.y = __builtin_bit_cast(float, w.z & 0xffff0000u) * m;
+                        hi.z = __builtin_bit_cast(float, w.w << 16) * m, hi.w = __builtin_bit_cast(float, w.w & 0xffff0000u) * m;
+                        *(f32x4*)dst = lo;
+                        *(f32x4*)(dst + 4) = hi;
+                    } else dst[0] = to_f32<T>(na[u]) * m;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UB; ++u) {
+                const int x = tid + u * LA_NT, j = x / CB, d = (x % CB) * WB;
+                if (j < TB && tn + j < t_hi) {
+                    if constexpr (VEC) *(f32x4*)(buf + j * per + 2 * Dp + d) = nb[u];
+                    else buf[j * per + 2 * Dp + d] = nb[u];
+                }
             }
         }
-        if (t0 + TB < t_hi) put(sm + (b ^ 1) * (TB * per), t0 + TB);
+        // the block's results leave after the next block's rows are in LDS: waiting for those loads does not wait for these stores
+        if (it >= 0 && dg == 0) {
+            const int n_tok = t_hi - t0 < TB ? t_hi - t0 : TB;
+            float* orow = out + ((size_t)t0 * H + h) * V + vcol;
+#pragma unroll
+            for (int j = 0; j < TB; ++j) {
+                if (j < n_tok && vok) orow[(size_t)j * H * V] = accs[j];
+                if (j < n_tok && vok2) orow[(size_t)j * H * V + 8] = accs2[j];
+            }
+        }
         __syncthreads();
     }
     if (keep) {
 #pragma unroll
         for (int r = 0; r < RR; ++r) {
-            const int d = dg * RR + r;
-            if (d < D) sm[d * (LA_VC + 1) + vc] = S[r];
+            const int d = LA_OWN(r);
+            if (d < D) sm[d * (LA_VC + 1) + vc] = S[r], sm[d * (LA_VC + 1) + vc + 8] = S2[r];
         }
         __syncthreads();
-        for (int i = tid; i < D * LA_VC; i += 256) {
+        for (int i = tid; i < D * LA_VC; i += LA_NT) {
             const int d = i / LA_VC, c = i % LA_VC;
             if (v0 + c < V) srow[(size_t)d * V + v0 + c] = sm[d * (LA_VC + 1) + c];
         }
     }
 }
+#undef LA_OWN
 
 struct la_args {
     dim3 grid; hipStream_t st; const void *q, *k, *v; int ldq, ldk, ldv; const float *decay, *head_decay; float q_scale;
     float* state; const int *cu_seqlens, *seq_slots; float* out; int H, D, V, keep;
 };
 
-template <typename T, int RR, bool CH, bool VEC>
+template <typename T, int RR, bool CH, bool VEC, int TB>
 static void la_launch(const la_args& a) {
-    constexpr int Dp = LA_DG * RR, per = (CH ? 3 : 2) * Dp + LA_VC, TB = la_block<RR>::tokens;
+    constexpr int Dp = LA_DG * RR, per = (CH ? 3 : 2) * Dp + LA_VC;
     constexpr size_t blocks = (size_t)2 * TB * per, tile = (size_t)Dp * (LA_VC + 1);
     constexpr size_t bytes = (blocks > tile ? blocks : tile) * sizeof(float);
     static_assert(bytes <= 64 * 1024, "linear_attn_scan: the token blocks must fit the default LDS limit");
-    linear_attn_scan_kernel<T, RR, CH, VEC><<<a.grid, 256, bytes, a.st>>>(
+    linear_attn_scan_kernel<T, RR, CH, VEC, TB><<<a.grid, LA_NT, bytes, a.st>>>(
         (const T*)a.q, (const T*)a.k, (const T*)a.v, a.ldq, a.ldk, a.ldv, a.decay, a.head_decay, a.q_scale, a.state, a.cu_seqlens,
         a.seq_slots, a.out, a.H, a.D, a.V, a.keep);
 }
 
-template <typename T, bool VEC>
-static void la_pick(const la_args& a) {
+template <typename T, bool VEC, int RR>
+static void la_pick_block(const la_args& a, bool single) {
+    constexpr int TB = la_block<RR>::tokens;
     const bool ch = a.decay != nullptr;
-    if (a.D <= 64) { if (ch) la_launch<T, 4, true, VEC>(a); else la_launch<T, 4, false, VEC>(a); }
-    else if (a.D <= 128) { if (ch) la_launch<T, 8, true, VEC>(a); else la_launch<T, 8, false, VEC>(a); }
-    else { if (ch) la_launch<T, 16, true, VEC>(a); else la_launch<T, 16, false, VEC>(a); }
+    if (single) { if (ch) la_launch<T, RR, true, VEC, 1>(a); else la_launch<T, RR, false, VEC, 1>(a); }
+    else { if (ch) la_launch<T, RR, true, VEC, TB>(a); else la_launch<T, RR, false, VEC, TB>(a); }
+}
+
+template <typename T, bool VEC>
+static void la_pick(const la_args& a, bool single) {
+    if (a.D <= 64) la_pick_block<T, VEC, 4>(a, single);
+    else if (a.D <= 128) la_pick_block<T, VEC, 8>(a, single);
+    else la_pick_block<T, VEC, 16>(a, single);
 }
 
 extern "C" int spite_linear_attn_scan(const void* q, const void* k, const void* v, int ldq, int ldk, int ldv, int dtype,
                                       const float* decay, const float* head_decay, float q_scale, float* state, int n_slots,
                                       const int* cu_seqlens, const int* seq_slots, int n_seqs, float* out,
-                                      int H, int D, int V, int keep, hipStream_t st) {
+                                      int H, int D, int V, int keep, int longest, hipStream_t st) {
     SP_REQUIRE(n_seqs >= 0 && H > 0 && D > 0 && V > 0 && n_slots > 0, "linear_attn_scan: bad sizes");
     SP_REQUIRE(D <= LA_MAXD, "linear_attn_scan: %d key channels a head (at most %d)", D, LA_MAXD);
     SP_REQUIRE(ldq >= H * D && ldk >= H * D && ldv >= H * V, "linear_attn_scan: rows shorter than the heads");
@@ -273,9 +285,10 @@ extern "C" int spite_linear_attn_scan(const void* q, const void* k, const void* 
     auto on16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
     const bool vec = dtype == SP_BF16 && D % 8 == 0 && V % 8 == 0 && ldq % 8 == 0 && ldk % 8 == 0 && ldv % 8 == 0
                      && on16(q) && on16(k) && on16(v) && on16(decay);
-    if (dtype == SP_F32) la_pick<float, false>(a);
-    else if (vec) la_pick<bf16, true>(a);
-    else la_pick<bf16, false>(a);
+    const bool single = longest == 1;               // (0: not known)
+    if (dtype == SP_F32) la_pick<float, false>(a, single);
+    else if (vec) la_pick<bf16, true>(a, single);
+    else la_pick<bf16, false>(a, single);
     SP_LAUNCH_CHECK("linear_attn_scan");
     return 0;
 }

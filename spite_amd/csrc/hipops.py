@@ -73,7 +73,7 @@ def lib():
             "spite_act_rows": [P, I, c_size_t, I, P],
             "spite_scale_rows": [P, c_size_t, F, P],
             "spite_channel_decay": [P, P, I, I, F, P],
-            "spite_linear_attn_scan": [P, P, P, I, I, I, I, P, P, F, P, I, P, P, I, P, I, I, I, I, P],
+            "spite_linear_attn_scan": [P, P, P, I, I, I, I, P, P, F, P, I, P, P, I, P, I, I, I, I, I, P],
             "spite_gated_group_norm": [P, P, I, P, I, P, I, I, I, I, F, I, P],
         }
         for name, args in sigs.items():
@@ -920,12 +920,13 @@ def _rows_view(t, name, width, T):
 
 
 def linear_attn_scan(q, k, v, out, state, cu_seqlens, seq_slots, n_seqs, H, D, V, *, decay=None, head_decay=None,
-                     q_scale=1.0, keep=True):
+                     q_scale=1.0, keep=True, longest=0):
     """The recurrence S = diag(a) S + k v^T, o = S^T q token by token for every entry of the step (see
     linear_attn.hip).  q, k [T, H*D] and v [T, H*V]: views of the run's dtype whose rows may lie apart;
     ``decay`` fp32 [T, H*D] (a number per key channel and token) or ``head_decay`` fp32 [H]; ``state`` fp32
     [slots, H, D, V], read at the entry's slot and, with ``keep``, left as the entry's last token leaves it;
-    out fp32 [T, H*V]."""
+    out fp32 [T, H*V].  ``longest``: the most tokens an entry has, if the caller knows (1 picks the kernel made
+    for single tokens; the results are the same bits either way)."""
     T = out.shape[0]
     if q.dtype != k.dtype or q.dtype != v.dtype:
         raise KernelError("linear_attn_scan: q, k and v of one dtype")
@@ -944,7 +945,7 @@ def linear_attn_scan(q, k, v, out, state, cu_seqlens, seq_slots, n_seqs, H, D, V
         pq, pk, pv, ldq, ldk, ldv, dtype_code(q.dtype), _ptr(decay, "decay", torch.float32, True),
         _ptr(head_decay, "head_decay", torch.float32, True), float(q_scale), _ptr(state, "state", torch.float32),
         state.shape[0], _ptr(cu_seqlens, "cu_seqlens", torch.int32), _ptr(seq_slots, "seq_slots", torch.int32), int(n_seqs),
-        _ptr(out, "out", torch.float32), H, D, V, int(bool(keep)), _stream()), "linear_attn_scan")
+        _ptr(out, "out", torch.float32), H, D, V, int(bool(keep)), int(longest), _stream()), "linear_attn_scan")
 
 
 NORM_GATES = {None: 0, "silu": 1, "sigmoid": 2}

@@ -137,7 +137,7 @@ class LinearAttention(Mixer):
         o = ws.take((T, HV), torch.float32)
         hipops.linear_attn_scan(qkv[:, :HD], qkv[:, HD:2 * HD], qkv[:, 2 * HD:2 * HD + HV], o, cache.state,
                                 ctx.cu_seqlens, ctx.seq_slots, ctx.n_seqs, H, D, V, decay=decay,
-                                head_decay=self.head_decay, q_scale=self.q_scale)
+                                head_decay=self.head_decay, q_scale=self.q_scale, longest=ctx.max_count)
         y = ws.take((T, HV), x.dtype)
         hipops.gated_group_norm(o, self.w_norm, y, V if self.out_norm == "head" else HV, self.eps,
                                 gate=rest[:, r:r + HV], act=self.gate)
