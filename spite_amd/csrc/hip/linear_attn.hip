@@ -321,6 +321,34 @@ void gated_group_norm_kernel(const float* __restrict__ o, const TO* __restrict__
     }
 }
 
+// The same for wide groups (the heads normed together): a workgroup a (token, group), the sum of squares across
+// its four waves through LDS.
+template <typename TO>
+__global__ __launch_bounds__(256)
+void gated_group_norm_wide_kernel(const float* __restrict__ o, const TO* __restrict__ gate, int ldg, const float* __restrict__ w,
+                                  int n_w, TO* __restrict__ y, int n, int group, float eps, int act) {
+    __shared__ float part[4];
+    const int groups = n / group;
+    const size_t t = blockIdx.x / groups;
+    const int c0 = (int)(blockIdx.x % groups) * group;
+    const float* orow = o + t * n + c0;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < group; c += 256) { const float x = orow[c]; ss = fmaf(x, x, ss); }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float sc = 1.0f / sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)group + eps);
+    for (int c = threadIdx.x; c < group; c += 256) {
+        float x = orow[c] * sc * w[(c0 + c) % n_w];
+        if (act) {
+            const float g = to_f32<TO>(gate[t * ldg + c0 + c]);
+            const float sg = 1.0f / (1.0f + expf(-g));
+            x *= act == 1 ? g * sg : sg;
+        }
+        y[t * n + c0 + c] = from_f32<TO>(x);
+    }
+}
+
 extern "C" int spite_gated_group_norm(const float* o, const void* gate, int ldg, const float* w, int n_w, void* y, int y_dtype,
                                       int T, int n, int group, float eps, int act, hipStream_t st) {
     SP_REQUIRE(T >= 0 && n > 0 && group > 0 && n % group == 0, "gated_group_norm: rows of %d in groups of %d", n, group);
@@ -330,6 +358,15 @@ extern "C" int spite_gated_group_norm(const float* o, const void* gate, int ldg,
     if (T == 0) return 0;
     const size_t items = (size_t)T * (n / group);
     SP_REQUIRE((items + 3) / 4 < (1u << 31), "gated_group_norm: too many groups");
+    if (group >= 512 && items < (1u << 31)) {
+        if (y_dtype == SP_F32)
+            gated_group_norm_wide_kernel<float><<<(unsigned)items, 256, 0, st>>>(o, (const float*)gate, ldg, w, n_w, (float*)y, n, group, eps, act);
+        else if (y_dtype == SP_BF16)
+            gated_group_norm_wide_kernel<bf16><<<(unsigned)items, 256, 0, st>>>(o, (const bf16*)gate, ldg, w, n_w, (bf16*)y, n, group, eps, act);
+        else return sp_fail("gated_group_norm: unknown dtype %d", y_dtype);
+        SP_LAUNCH_CHECK("gated_group_norm");
+        return 0;
+    }
     const unsigned grid = (unsigned)((items + 3) / 4);
     if (y_dtype == SP_F32)
         gated_group_norm_kernel<float><<<grid, 256, 0, st>>>(o, (const float*)gate, ldg, w, n_w, (float*)y, T, n, group, eps, act);

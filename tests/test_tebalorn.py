@@ -362,7 +362,7 @@ def test_channel_decay_kernel(tau):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n,group,n_w,act", [(30, 10, 10, "silu"), (24, 24, 24, "sigmoid"), (256, 128, 128, "silu"), (96, 96, 96, None)])
+@pytest.mark.parametrize("n,group,n_w,act", [(30, 10, 10, "silu"), (24, 24, 24, "sigmoid"), (256, 128, 128, "silu"), (96, 96, 96, None), (1300, 1300, 1300, "sigmoid"), (2048, 1024, 1024, "silu")])
 def test_norm_and_gate_kernel(dtype, n, group, n_w, act):
     from spite_amd.csrc import hipops
     g = torch.Generator().manual_seed(n)
