@@ -255,11 +255,11 @@ def pefedra_configs(sz, layers, window, vocab):
 def tebalorn_configs(sz, layers, window, vocab):
     H = sz["heads"]
     linear = {"heads": H, "dim": 128, "vdim": 128}
-    mixers = [("gla", dict(linear, tau=16.0)),
+    mixers = [("gla", dict(linear, tau=8.0)),
               ("lightning", dict(linear, decay=[1.0 - 2.0 ** (-5.0 - 3.0 * h / max(H - 1, 1)) for h in range(H)])),
               ("attention", {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
                              "mask": {"size": window},
-                             "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}),
+                             "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 8192, "fast": 16.0, "slow": 2.0}}}),
               ("lightning", dict(linear, decay=[1.0 - 2.0 ** (-4.0 - 4.0 * h / max(H - 1, 1)) for h in range(H)]))]
     mlp = {"kind": "moe", "router": {"experts": sz["experts"], "top": sz["top"]}, "expert": {"ff": sz["expert_ff"]},
            "shared": {"ff": sz["shared_ff"]}}
