@@ -38,20 +38,21 @@ extern "C" int spite_channel_decay(float* z, const float* bias, int T, int width
 }
 
 // ------------------------------------------------------------------ the recurrence, token by token
-// A workgroup of 128 threads takes 16 value columns of one head of one entry of the step and walks the
-// entry's tokens in order.  Thread (vc, dg) = (tid / 16, tid % 16) holds, in registers, the state's elements
-// S[d][v0 + vc] and S[d][v0 + vc + 8] for the key channels d = 64 m + 4 dg + x (x < 4, m < RR / 4; RR = 4, 8 or
-// 16 for up to 64, 128 or 256 key channels): 16 lanes read 256 consecutive bytes of a token's q, k or decay
-// row from LDS in one wide read without bank conflicts, and every such read serves two columns (LDS reads,
-// not FMAs, bound the walk).  The tokens' q, k, decay and value slice go through LDS a block of tokens at a
-// time, two buffers: the next block's loads are in flight while this block is computed, and a whole block is
-// one stretch of code: only the state's FMA waits for the token before.  The sum over the key channels is a
-// thread's own partial sum and four rotations across its 16 neighbours.  The state tile goes through LDS on
-// the way in and out, so that its rows are read and written 64 bytes at a time.
+// A workgroup of 512 threads takes 16 value columns of one head of one entry of the step and walks the
+// entry's tokens in order.  Thread (vc, dg) = (tid / 32, tid % 32) holds, in registers, the state's elements
+// S[d][v0 + vc] and S[d][v0 + vc + 8] for D / 32 key channels d (four consecutive ones at 4 dg, and again 128
+// further on for the widest heads; two at 2 dg for heads up to 64): 32 lanes read 512 consecutive bytes of a
+// token's q, k or decay row from LDS in one wide read without bank conflicts.  The tokens' q, k, decay and value slice go through LDS a block of tokens at a time, two buffers:
+// the next block's loads are in flight while this block is computed, and a whole block is one stretch of code:
+// only the state's FMA waits for the token before.  The sum over the key channels is a thread's own partial
+// sum, four rotations across a row of 16 lanes and one step from the lower row to the upper.  The state tile
+// goes through LDS on the way in and out, so that its rows are read and written 64 bytes at a time.
+// The walk is bound by latency, not by FMAs or bytes (about a third of a SIMD's issue slots are used): the
+// split over 32 lanes a column is there to have more waves to switch between.
 // The order of every sum is fixed by D alone: the bits do not depend on how a request's tokens are cut.
 #define LA_VC 16        // value columns a workgroup
-#define LA_NT 128       // threads a workgroup: 8 x 16, two columns a thread
-#define LA_DG 16
+#define LA_NT 512       // threads a workgroup: 16 columns x 32 lanes
+#define LA_DG 32        // lanes that share a column's key channels
 #define LA_MAXD 256
 
 template <int RR> struct la_block { static constexpr int tokens = RR == 16 ? 8 : 16; };
@@ -67,9 +68,16 @@ __device__ __forceinline__ float row16_sum(float x) {
     return x;
 }
 
+// The sum over 32 lanes (two rows of 16): the rows' sums, then the lower row's into the upper row (a row's last
+// lane to the next row, rows 1 and 3 only).  The upper 16 of the 32 lanes get it.
+__device__ __forceinline__ float row32_sum(float x) {
+    x = row16_sum(x);
+    return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
+}
+
 // VEC: q, k, v (bfloat16) and the decay rows start on 16 bytes and D and V are multiples of 8: a fetch is
 // 16 bytes.  Otherwise one element.  (Plain loops and no closures: every array below stays in registers.)
-#define LA_OWN(r) (((r) / 4) * 64 + dg * 4 + ((r) % 4))          // the thread's r-th key channel
+#define LA_OWN(r) (PR >= 4 ? ((r) / 4) * 128 + dg * 4 + ((r) % 4) : dg * PR + (r))    // the thread's r-th key channel
 // TB: tokens a block: 16 (8 for the widest heads), or 1 for steps of single tokens, whose workgroups then hold
 // little LDS and few registers, so that many are resident and their round trips to memory overlap.
 template <typename T, int RR, bool CH, bool VEC, int TB>
@@ -78,7 +86,8 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
                              const float* __restrict__ decay, const float* __restrict__ head_decay, float q_scale,
                              float* __restrict__ state, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots,
                              float* __restrict__ out, int H, int D, int V, int keep) {
-    constexpr int Dp = LA_DG * RR;                  // key channels, padded
+    constexpr int Dp = 16 * RR;                     // key channels, padded
+    constexpr int PR = RR / 2;                      // key channels a thread
     constexpr int NQ = CH ? 3 : 2;                  // rows of Dp a token: q, k and, per channel, the decay
     constexpr int per = NQ * Dp + LA_VC;
     // A fetch is one load and no branch around it.  Two lists of fetches a block: A from q, k and the value
@@ -88,6 +97,8 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
     constexpr int UA = (TB * CA + LA_NT - 1) / LA_NT, UB = CH ? (TB * CB + LA_NT - 1) / LA_NT : 0;   // fetches a thread and block
     typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
     typedef float f32x4 __attribute__((ext_vector_type(4)));
+    constexpr int PV = PR < 4 ? PR : 4;             // key channels an LDS read
+    typedef float vec __attribute__((ext_vector_type(PV)));
     using RawA = typename std::conditional<VEC, u32x4, T>::type;
     using RawB = typename std::conditional<VEC, f32x4, float>::type;
     extern __shared__ __attribute__((aligned(16))) float sm[];      // max(2 * TB * per, Dp * 17) floats
@@ -95,20 +106,19 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
     const int tid = threadIdx.x, vc = tid / LA_DG, dg = tid % LA_DG;
     const int t_lo = cu_seqlens[e], t_hi = cu_seqlens[e + 1];
     if (t_lo >= t_hi) return;
-    const int vcol = v0 + vc;                       // and vcol + 8
-    const bool vok = vcol < V, vok2 = vcol + 8 < V;
+    const int vcol = v0 + vc;
+    const bool vok = vcol < V;
     float* srow = state + ((size_t)seq_slots[e] * H + h) * (size_t)D * V;
     for (int i = tid; i < D * LA_VC; i += LA_NT) {
         const int d = i / LA_VC, c = i % LA_VC;
         sm[d * (LA_VC + 1) + c] = v0 + c < V ? srow[(size_t)d * V + v0 + c] : 0.f;
     }
     __syncthreads();
-    float S[RR], S2[RR];
+    float S[PR];
 #pragma unroll
-    for (int r = 0; r < RR; ++r) {
+    for (int r = 0; r < PR; ++r) {
         const int d = LA_OWN(r);
         S[r] = d < D ? sm[d * (LA_VC + 1) + vc] : 0.f;
-        S2[r] = d < D ? sm[d * (LA_VC + 1) + vc + 8] : 0.f;
     }
     __syncthreads();
     const float hd = CH ? 1.f : head_decay[h];
@@ -140,7 +150,7 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
                 nb[u] = ok ? got : RawB{};
             }
         }
-        float accs[TB], accs2[TB];
+        float accs[TB];
         if (it >= 0) {
             const float* cur = sm + (it & 1) * (TB * per);
             const int n_tok = t_hi - t0 < TB ? t_hi - t0 : TB;
@@ -150,20 +160,19 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
 #define LA_TOKEN(j)                                                                         \
             {                                                                               \
                 const float* row = cur + (j) * per;                                         \
-                const float vv = row[NQ * Dp + vc], vv2 = row[NQ * Dp + vc + 8];            \
-                accs[j] = accs2[j] = 0.f;                                                   \
+                const float vv = row[NQ * Dp + vc];                                         \
+                accs[j] = 0.f;                                                              \
                 _Pragma("unroll")                                                           \
-                for (int r = 0; r < RR; r += 4) {                                           \
-                    const f32x4 q4 = *(const f32x4*)(row + LA_OWN(r));                      \
-                    const f32x4 k4 = *(const f32x4*)(row + Dp + LA_OWN(r));                 \
-                    f32x4 a4 = {hd, hd, hd, hd};                                            \
-                    if (CH) a4 = *(const f32x4*)(row + 2 * Dp + LA_OWN(r));                 \
+                for (int r = 0; r < PR; r += PV) {                                          \
+                    const vec q4 = *(const vec*)(row + LA_OWN(r));                          \
+                    const vec k4 = *(const vec*)(row + Dp + LA_OWN(r));                     \
+                    vec a4;                                                                 \
+                    if (CH) a4 = *(const vec*)(row + 2 * Dp + LA_OWN(r));                   \
                     _Pragma("unroll")                                                       \
-                    for (int y = 0; y < 4; ++y) {                                           \
-                        S[r + y] = fmaf(a4[y], S[r + y], k4[y] * vv);                       \
-                        S2[r + y] = fmaf(a4[y], S2[r + y], k4[y] * vv2);                    \
+                    for (int y = 0; y < PV; ++y) {                                          \
+                        const float a = CH ? a4[y] : hd;                                    \
+                        S[r + y] = fmaf(a, S[r + y], k4[y] * vv);                           \
                         accs[j] = fmaf(S[r + y], q4[y], accs[j]);                           \
-                        accs2[j] = fmaf(S2[r + y], q4[y], accs2[j]);                        \
                     }                                                                       \
                 }                                                                           \
             }
@@ -174,13 +183,13 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
             } else {
 #pragma unroll
                 for (int j = 0; j < TB; ++j) {
-                    accs[j] = accs2[j] = 0.f;
+                    accs[j] = 0.f;
                     if (j < n_tok) LA_TOKEN(j)
                 }
             }
 #undef LA_TOKEN
 #pragma unroll
-            for (int j = 0; j < TB; ++j) accs[j] = row16_sum(accs[j]), accs2[j] = row16_sum(accs2[j]);
+            for (int j = 0; j < TB; ++j) accs[j] = row32_sum(accs[j]);
         }
         if (more) {
             float* buf = sm + ((it + 1) & 1) * (TB * per);
@@ -212,22 +221,21 @@ void linear_attn_scan_kernel(const T* __restrict__ q, const T* __restrict__ k, c
             }
         }
         // the block's results leave after the next block's rows are in LDS: waiting for those loads does not wait for these stores
-        if (it >= 0 && dg == 0) {
+        if (it >= 0 && dg == LA_DG - 1) {
             const int n_tok = t_hi - t0 < TB ? t_hi - t0 : TB;
             float* orow = out + ((size_t)t0 * H + h) * V + vcol;
 #pragma unroll
             for (int j = 0; j < TB; ++j) {
                 if (j < n_tok && vok) orow[(size_t)j * H * V] = accs[j];
-                if (j < n_tok && vok2) orow[(size_t)j * H * V + 8] = accs2[j];
             }
         }
         __syncthreads();
     }
     if (keep) {
 #pragma unroll
-        for (int r = 0; r < RR; ++r) {
+        for (int r = 0; r < PR; ++r) {
             const int d = LA_OWN(r);
-            if (d < D) sm[d * (LA_VC + 1) + vc] = S[r], sm[d * (LA_VC + 1) + vc + 8] = S2[r];
+            if (d < D) sm[d * (LA_VC + 1) + vc] = S[r];
         }
         __syncthreads();
         for (int i = tid; i < D * LA_VC; i += LA_NT) {
@@ -245,7 +253,7 @@ struct la_args {
 
 template <typename T, int RR, bool CH, bool VEC, int TB>
 static void la_launch(const la_args& a) {
-    constexpr int Dp = LA_DG * RR, per = (CH ? 3 : 2) * Dp + LA_VC;
+    constexpr int Dp = 16 * RR, per = (CH ? 3 : 2) * Dp + LA_VC;
     constexpr size_t blocks = (size_t)2 * TB * per, tile = (size_t)Dp * (LA_VC + 1);
     constexpr size_t bytes = (blocks > tile ? blocks : tile) * sizeof(float);
     static_assert(bytes <= 64 * 1024, "linear_attn_scan: the token blocks must fit the default LDS limit");
