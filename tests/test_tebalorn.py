@@ -6,6 +6,9 @@ from __future__ import annotations
 
 import copy
 import math
+import os
+import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -781,3 +784,22 @@ def test_replay_program(models):
     ref = plain_rows(cfg, weights, reqs)
     err, where = H.max_diff(got, ref)
     assert err <= 2e-4 * scale_of(ref), f"{err} at {where}"
+
+
+@pytest.mark.gpu
+def test_command_line_and_sampling(models):
+    """`spite run` on the model's folder: the greedy tokens of `Engine.generate`; and sampling with a seed through
+    the framework's sampler gives the same tokens twice and other tokens than greedy somewhere."""
+    cfg = CONFIGS["small"]
+    folder, _ = models("small", "float32")
+    p = H.random_tokens(cfg["vocab"], 9, 21)
+    eng = engine(folder, "float32", "small", cache_tokens=256)
+    want = eng.generate([p], max_tokens=12, temperature=0.0)[0]
+    out = subprocess.run([sys.executable, os.path.join(H.ROOT, "bin", "spite"), "run", "-m", str(folder), "--prompt-ids",
+                          ",".join(map(str, p)), "--max-tokens", "12", "--temperature", "0", "--dtype", "fp32",
+                          "--ctx", "64", "--page-size", "16"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.strip().splitlines()[-1].split() == [str(t) for t in want]
+    a = eng.generate([p, p[:4]], max_tokens=12, temperature=1.0, seed=5)
+    b = eng.generate([p, p[:4]], max_tokens=12, temperature=1.0, seed=5)
+    assert a == b and a[0] != want
