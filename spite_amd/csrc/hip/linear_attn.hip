@@ -341,13 +341,16 @@ void gated_group_norm_wide_kernel(const float* __restrict__ o, const TO* __restr
     const int c0 = (int)(blockIdx.x % groups) * group;
     const float* orow = o + t * n + c0;
     float ss = 0.f;
+#pragma unroll 8
     for (int c = threadIdx.x; c < group; c += 256) { const float x = orow[c]; ss = fmaf(x, x, ss); }
     ss = wave_sum(ss);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
     const float sc = 1.0f / sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)group + eps);
+    const bool whole = n_w >= n;                      // a weight for every element of the row: no wrapping
+#pragma unroll 4
     for (int c = threadIdx.x; c < group; c += 256) {
-        float x = orow[c] * sc * w[(c0 + c) % n_w];
+        float x = orow[c] * sc * w[whole ? c0 + c : (c0 + c) % n_w];
         if (act) {
             const float g = to_f32<TO>(gate[t * ldg + c0 + c]);
             const float sg = 1.0f / (1.0f + expf(-g));
