@@ -14,6 +14,7 @@
 #include "common.h"
 
 #define WIDE_NT 256
+#define QKV_MAX_HPB 16     // heads a workgroup of qkv_prepare, at most
 
 // ------------------------------------------------------------------ projection row -> q, cache
 // A workgroup takes `hpb` heads of one token (query heads first, then key heads, then value heads; with
@@ -35,7 +36,8 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
                         T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
                         const int* __restrict__ positions, const int* __restrict__ slot_map,
                         const float* __restrict__ inv_freq, int rot, float rot_mag, const float* __restrict__ inv_freq_v,
-                        int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp, int hpb) {
+                        int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp, int hpb,
+                        int head_norm, float qt_coef, int qt_every, int v_from_k) {
     extern __shared__ float sm[];
     __shared__ float red[WIDE_NT / 64];
     const int rh = rot >> 1, vh = inv_freq_v ? (Vd >> 1) : 0;
@@ -57,12 +59,24 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
     const int v_lo = (h_lo > HQ + GK ? h_lo : HQ + GK) - (HQ + GK);
     const int v_hi = (h_end < HQ + GK + GV ? h_end : HQ + GK + GV) - (HQ + GK);       // value heads [v_lo, v_hi)
     float scale_q = 1.f, scale_k = 1.f;
-    if (wq && h_lo < HQ) {
+    __shared__ float head_sc[QKV_MAX_HPB];
+    if (head_norm) {
+        // a norm per head: a wave forms the sum of squares of one head of this workgroup at a time
+        for (int hh = h_lo + (tid >> 6); hh < qk_hi; hh += WIDE_NT / 64) {
+            float s = 0.f;
+            for (int c = tid & 63; c < D; c += 64) { const float x = to_f32<T>(row[hh * D + c]) + (bias ? bias[hh * D + c] : 0.f); s += x * x; }
+            s = wave_sum(s);
+            if ((tid & 63) == 0) head_sc[hh - h_lo] = 1.0f / sqrtf(s / (float)D + eps);
+        }
+    }
+    // the query's temperature: a factor that grows with the logarithm of the position, in steps
+    const float q_temp = qt_every > 0 ? 1.0f + qt_coef * logf((float)((positions[t] + 1) / qt_every) + 1.0f) : 1.0f;
+    if (!head_norm && wq && h_lo < HQ) {
         float s = 0.f;
         for (int c = tid; c < Nq; c += WIDE_NT) { const float x = to_f32<T>(row[c]) + (bias ? bias[c] : 0.f); s += x * x; }
         scale_q = 1.0f / sqrtf(block_sum<WIDE_NT>(s, red) / (float)Nq + eps);
     }
-    if (wk && h_lo < qk_end && h_end > HQ) {
+    if (!head_norm && wk && h_lo < qk_end && h_end > HQ) {
         float s = 0.f;
         for (int c = tid; c < Nk; c += WIDE_NT) { const float x = to_f32<T>(row[Nq + c]) + (bias ? bias[Nq + c] : 0.f); s += x * x; }
         scale_k = 1.0f / sqrtf(block_sum<WIDE_NT>(s, red) / (float)Nk + eps);
@@ -78,12 +92,13 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
         const bool is_q = hh < HQ;
         const int base = hh * D;                       // the q and k regions follow each other in the row
         const float* wn = is_q ? wq : wk;
-        const float sc = is_q ? scale_q : scale_k;
-        const int wbase = is_q ? base : base - Nq;
+        const float sc = head_norm ? head_sc[hh - h_lo] : (is_q ? scale_q : scale_k);
+        const int wbase = head_norm ? 0 : (is_q ? base : base - Nq);      // a head norm's weights serve every head
+        const float qt = is_q ? q_temp : 1.0f;
         auto load = [&](int c) {
             float x = to_f32<T>(row[base + c]) + (bias ? bias[base + c] : 0.f);
             if (wn) x = x * sc * wn[wbase + c];
-            return x;
+            return x * qt;
         };
         T* dst = nullptr;
         if (is_q) dst = q_out + ((size_t)t * HQ + hh) * Dp;
@@ -108,7 +123,7 @@ void qkv_prepare_kernel(const T* __restrict__ qkv, int ld, const float* __restri
     }
     if (slot < 0) return;
     const int vitems = Vd - vh;
-    const int vbase = Nq + Nk;
+    const int vbase = v_from_k ? Nq : Nq + Nk;           // the values are the keys as the row holds them (before their norm)
     for (int it = tid; it < (v_hi > v_lo ? v_hi - v_lo : 0) * vitems; it += WIDE_NT) {
         const int g = v_lo + it / vitems, i = it % vitems;
         T* slab = v_pages + (page * GV + g) * (size_t)Vd * ps;
@@ -134,7 +149,8 @@ void qkv_prepare_vec_kernel(const bf16* __restrict__ qkv, int ld, const float* _
                             bf16* __restrict__ q_out, bf16* __restrict__ k_pages, bf16* __restrict__ v_pages,
                             const int* __restrict__ positions, const int* __restrict__ slot_map,
                             const float* __restrict__ inv_freq, int rot, float rot_mag, const float* __restrict__ inv_freq_v,
-                            int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp, int hpb) {
+                            int HQ, int GK, int GV, int D, int Vd, int ps, int k_tiled, int v_tiled, int Dp, int hpb,
+                            int head_norm, float qt_coef, int qt_every, int v_from_k) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
     __shared__ float red[WIDE_NT / 64];
     const int rh = rot >> 1, vh = inv_freq_v ? (Vd >> 1) : 0;
@@ -166,8 +182,18 @@ void qkv_prepare_vec_kernel(const bf16* __restrict__ qkv, int ld, const float* _
         return block_sum<WIDE_NT>(s, red);
     };
     float scale_q = 1.f, scale_k = 1.f;
-    if (wq && h_lo < HQ) scale_q = 1.0f / sqrtf(sumsq(0, Nq) / (float)Nq + eps);
-    if (wk && h_lo < qk_end && h_end > HQ) scale_k = 1.0f / sqrtf(sumsq(Nq, Nk) / (float)Nk + eps);
+    __shared__ float head_sc[QKV_MAX_HPB];
+    if (head_norm) {
+        for (int hh = h_lo + (tid >> 6); hh < qk_hi; hh += WIDE_NT / 64) {
+            float s = 0.f;
+            for (int c = (tid & 63) * 4; c < D; c += 256) { const f32x4 x = row4(hh * D + c); s += x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3]; }
+            s = wave_sum(s);
+            if ((tid & 63) == 0) head_sc[hh - h_lo] = 1.0f / sqrtf(s / (float)D + eps);
+        }
+    }
+    const float q_temp = qt_every > 0 ? 1.0f + qt_coef * logf((float)((positions[t] + 1) / qt_every) + 1.0f) : 1.0f;
+    if (!head_norm && wq && h_lo < HQ) scale_q = 1.0f / sqrtf(sumsq(0, Nq) / (float)Nq + eps);
+    if (!head_norm && wk && h_lo < qk_end && h_end > HQ) scale_k = 1.0f / sqrtf(sumsq(Nq, Nk) / (float)Nk + eps);
     __syncthreads();
     const size_t page = slot >= 0 ? (size_t)(slot / ps) : 0;
     const int off = slot >= 0 ? slot % ps : 0;
@@ -179,12 +205,13 @@ void qkv_prepare_vec_kernel(const bf16* __restrict__ qkv, int ld, const float* _
         const bool is_q = hh < HQ;
         const int base = hh * D;
         const float* wn = is_q ? wq : wk;
-        const float sc = is_q ? scale_q : scale_k;
-        const int wbase = is_q ? base : base - Nq;
+        const float sc = head_norm ? head_sc[hh - h_lo] : (is_q ? scale_q : scale_k);
+        const int wbase = head_norm ? 0 : (is_q ? base : base - Nq);
+        const float qt = is_q ? q_temp : 1.0f;
         auto load = [&](int c) {
             f32x4 x = row4(base + c);
             if (wn) { const f32x4 ww = *(const f32x4*)(wn + wbase + c); x = x * sc * ww; }
-            return x;
+            return x * qt;
         };
         bf16* dst = is_q ? q_out + ((size_t)t * HQ + hh) * Dp : k_pages + (page * GK + (hh - HQ)) * (size_t)ps * Dp;
         auto store = [&](int c, const f32x4& v) {
@@ -206,7 +233,7 @@ void qkv_prepare_vec_kernel(const bf16* __restrict__ qkv, int ld, const float* _
     }
     if (slot < 0) return;
     const int vitems = Vd - vh;
-    const int vbase = Nq + Nk;
+    const int vbase = v_from_k ? Nq : Nq + Nk;
     for (int it = tid; it < (v_hi > v_lo ? v_hi - v_lo : 0) * vitems; it += WIDE_NT) {
         const int g = v_lo + it / vitems, i = it % vitems;
         bf16* slab = v_pages + (page * GV + g) * (size_t)Vd * ps;
@@ -226,11 +253,14 @@ extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float
                                  float eps, void* q_out, void* k_pages, void* v_pages, const int* positions,
                                  const int* slot_map, const float* inv_freq, int rot, float rot_mag, const float* inv_freq_v,
                                  int T, int HQ, int GK, int GV, int D, int Vd, int page_size, int k_tiled, int v_tiled,
-                                 int Dp, hipStream_t st) {
+                                 int Dp, int head_norm, float qt_coef, int qt_every, int v_from_k, hipStream_t st) {
     if (Dp <= 0) Dp = D;
     SP_REQUIRE(Dp >= D, "qkv_prepare: heads of %d stored with %d elements", D, Dp);
     SP_REQUIRE(T >= 0 && HQ > 0 && GK > 0 && GV > 0 && D > 0 && Vd > 0 && page_size > 0, "qkv_prepare: bad sizes");
-    SP_REQUIRE(ld >= (HQ + GK) * D + GV * Vd, "qkv_prepare: rows of %d elements for %d", ld, (HQ + GK) * D + GV * Vd);
+    SP_REQUIRE(ld >= (HQ + GK) * D + (v_from_k ? 0 : GV * Vd), "qkv_prepare: rows of %d elements for %d", ld, (HQ + GK) * D + (v_from_k ? 0 : GV * Vd));
+    SP_REQUIRE(!v_from_k || (GV == GK && Vd == D && !inv_freq_v), "qkv_prepare: values taken from the keys have the keys' heads and width");
+    SP_REQUIRE(!head_norm || (wq && wk), "qkv_prepare: a head norm needs its two weight vectors");
+    SP_REQUIRE(qt_every >= 0, "qkv_prepare: query temperature every %d positions", qt_every);
     SP_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D, "qkv_prepare: %d turning elements of a head of %d", rot, D);
     SP_REQUIRE(rot == 0 || inv_freq, "qkv_prepare: rotation needs a frequency table");
     SP_REQUIRE(!inv_freq_v || Vd % 2 == 0, "qkv_prepare: values of %d elements cannot turn in pairs", Vd);
@@ -245,7 +275,7 @@ extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float
     const int heads = HQ + GK + GV;
     long hpb = ((long)heads * T + 2 * sp_cu_count() - 1) / (2 * sp_cu_count());
     if (hpb < 1) hpb = 1;
-    if (hpb > 16) hpb = 16;                          // (more waves in flight hide the rows' 2-byte loads and stores)
+    if (hpb > QKV_MAX_HPB) hpb = QKV_MAX_HPB;                          // (more waves in flight hide the rows' 2-byte loads and stores)
     if (hpb > heads) hpb = heads;
     const dim3 grid(T, (unsigned)((heads + hpb - 1) / hpb));
     auto al = [](const void* p, int a) { return ((uintptr_t)p & (a - 1)) == 0; };
@@ -253,16 +283,16 @@ extern "C" int spite_qkv_prepare(const void* qkv, int ld, int dtype, const float
         && al(bias, 16) && al(wq, 16) && al(wk, 16)) {
         // (the sine and cosine tables are read four at a time: the second starts rot/2 floats behind the first)
         qkv_prepare_vec_kernel<<<grid, WIDE_NT, sh, st>>>((const bf16*)qkv, ld, bias, wq, wk, eps, (bf16*)q_out, (bf16*)k_pages,
-            (bf16*)v_pages, positions, slot_map, inv_freq, rot, rot_mag, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
+            (bf16*)v_pages, positions, slot_map, inv_freq, rot, rot_mag, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb, head_norm, qt_coef, qt_every, v_from_k);
         SP_LAUNCH_CHECK("qkv_prepare");
         return 0;
     }
     if (dtype == SP_F32)
         qkv_prepare_kernel<float><<<grid, WIDE_NT, sh, st>>>((const float*)qkv, ld, bias, wq, wk, eps, (float*)q_out, (float*)k_pages,
-            (float*)v_pages, positions, slot_map, inv_freq, rot, rot_mag, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
+            (float*)v_pages, positions, slot_map, inv_freq, rot, rot_mag, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb, head_norm, qt_coef, qt_every, v_from_k);
     else if (dtype == SP_BF16)
         qkv_prepare_kernel<bf16><<<grid, WIDE_NT, sh, st>>>((const bf16*)qkv, ld, bias, wq, wk, eps, (bf16*)q_out, (bf16*)k_pages,
-            (bf16*)v_pages, positions, slot_map, inv_freq, rot, rot_mag, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb);
+            (bf16*)v_pages, positions, slot_map, inv_freq, rot, rot_mag, inv_freq_v, HQ, GK, GV, D, Vd, page_size, k_tiled, v_tiled, Dp, (int)hpb, head_norm, qt_coef, qt_every, v_from_k);
     else return sp_fail("qkv_prepare: unknown dtype %d", dtype);
     SP_LAUNCH_CHECK("qkv_prepare");
     return 0;
@@ -282,7 +312,7 @@ void attn_wide_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
                       TO* __restrict__ out, const int* __restrict__ positions,
                       const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                       int max_blocks, int HQ, int GK, int GV, int D, int Vd, int ps, int vis, int span, float scale,
-                      int k_tiled, int v_tiled, const float* __restrict__ sinks) {
+                      int k_tiled, int v_tiled, const float* __restrict__ sinks, const float* __restrict__ slopes) {
     extern __shared__ float smem[];
     float* q_sh = smem;                 // [D]
     float* p_sh = smem + D;             // [64]
@@ -316,6 +346,7 @@ void attn_wide_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
                 float acc = 0.f;
                 for (int c = 0; c < D; ++c) acc = fmaf(q_sh[c], to_f32<T>(kr[sp_k_index(j % ps, c, D, k_tiled)]), acc);
                 s = acc * scale;
+                if (slopes) s += slopes[h] * (float)(j - p);       // a bias that grows with the distance
             }
         }
         const float m_new = fmaxf(m, wave_max(s));
@@ -355,7 +386,7 @@ void attn_wide_kernel(const T* __restrict__ q, const T* __restrict__ k_pages, co
 extern "C" int spite_attn_wide(const void* q, const void* k_pages, const void* v_pages, void* out, int dtype, int out_dtype,
                                const int* positions, const int* seq_of_token, const int* block_table,
                                int max_blocks, int T, int HQ, int GK, int GV, int D, int Vd, int page_size, int vis, int span,
-                               float scale, int k_tiled, int v_tiled, const float* sinks, hipStream_t st) {
+                               float scale, int k_tiled, int v_tiled, const float* sinks, const float* slopes, hipStream_t st) {
     SP_REQUIRE(T >= 0 && HQ > 0 && GK > 0 && GV > 0 && HQ % GK == 0 && GK % GV == 0,
                "attention: %d query heads over %d key heads over %d value heads", HQ, GK, GV);
     SP_REQUIRE(D > 0 && D <= 4096 && Vd > 0 && Vd <= 64 * WIDE_MAX_V, "attention: keys of %d, values of %d (at most %d)", D, Vd, 64 * WIDE_MAX_V);
@@ -368,7 +399,7 @@ extern "C" int spite_attn_wide(const void* q, const void* k_pages, const void* v
     dim3 grid(T, HQ);
     const size_t sh = (size_t)(D + 64) * sizeof(float) + 128 * sizeof(int);
 #define SP_AW(TI, TO) attn_wide_kernel<TI, TO><<<grid, 64, sh, st>>>((const TI*)q, (const TI*)k_pages, (const TI*)v_pages, (TO*)out, \
-        positions, seq_of_token, block_table, max_blocks, HQ, GK, GV, D, Vd, page_size, vis, span, scale, k_tiled, v_tiled, sinks)
+        positions, seq_of_token, block_table, max_blocks, HQ, GK, GV, D, Vd, page_size, vis, span, scale, k_tiled, v_tiled, sinks, slopes)
     if (dtype == SP_F32 && out_dtype == SP_F32) SP_AW(float, float);
     else if (dtype == SP_BF16 && out_dtype == SP_BF16) SP_AW(bf16, bf16);
     else if (dtype == SP_BF16 && out_dtype == SP_F32) SP_AW(bf16, float);

@@ -143,12 +143,12 @@ __device__ __forceinline__ float sp_gate_act(float g, int act, bool fast) {
 }
 
 // An activation on its own (no gate): SP_UNARY_GELU 0.5 z (1 + erf(z / sqrt 2)), SP_UNARY_GELU_TANH,
-// SP_UNARY_SILU, in fp32.  `fast` (the bfloat16 products' epilogues): the short exponential, and for the
+// SP_UNARY_SILU, SP_UNARY_TANH, in fp32.  `fast` (the bfloat16 products' epilogues): the short exponential, and for the
 // error function the rational form 1 - (a1 t + ... + a5 t^5) exp(-x^2), t = 1 / (1 + p x), whose error of
 // 1.5e-7 is a thousandth of a bfloat16 step; else the accurate routines.  The product kernels take one as
 // the epilogue of a plain product: their `glu` argument carries it in the bits above the gate's code
 // (glu = unary << 4).
-enum { SP_UNARY_GELU = 1, SP_UNARY_GELU_TANH = 2, SP_UNARY_SILU = 3 };
+enum { SP_UNARY_GELU = 1, SP_UNARY_GELU_TANH = 2, SP_UNARY_SILU = 3, SP_UNARY_TANH = 4 };
 __device__ __forceinline__ float sp_unary(float z, int act, bool fast) {
     if (act == SP_UNARY_GELU) {
         if (!fast) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
@@ -158,6 +158,7 @@ __device__ __forceinline__ float sp_unary(float z, int act, bool fast) {
         const float e = 1.0f - poly * __expf(-x * x);              // erf(|z| / sqrt 2)
         return 0.5f * z * (1.0f + copysignf(e, z));
     }
+    if (act == SP_UNARY_TANH) return fast ? 1.0f - 2.0f / (__expf(2.0f * z) + 1.0f) : tanhf(z);
     if (act == SP_UNARY_GELU_TANH) return sp_gate_act(z, SP_ACT_GELU_TANH, fast);
     return sp_gate_act(z, SP_ACT_SILU, fast);
 }

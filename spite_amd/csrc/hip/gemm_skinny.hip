@@ -204,7 +204,7 @@ extern "C" int spite_gemm_skinny(const void* X, int ldx, const void* W, long w_g
     SP_REQUIRE(M >= 0 && N > 0 && K > 0 && ldx >= K && ldy >= N, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
     const int unary = glu >> 4;
     glu &= 15;
-    SP_REQUIRE(!(glu && unary) && unary <= SP_UNARY_SILU, "gemm_skinny: activation code %d", glu | (unary << 4));
+    SP_REQUIRE(!(glu && unary) && unary <= SP_UNARY_TANH, "gemm_skinny: activation code %d", glu | (unary << 4));
     g_skinny_act = glu ? glu : -unary;
     SP_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny: K=%d and the row stride %d must be multiples of 8", K, ldx);
     SP_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_skinny: operands must be 16-byte aligned");

@@ -400,7 +400,7 @@ extern "C" int spite_gemm_tiled(const void* X, int ldx, const void* W, long w_gr
     SP_REQUIRE(shape >= 0 && shape <= 6, "gemm_tiled: tile shape %d", shape);
     const int unary = glu >> 4;
     glu &= 15;
-    SP_REQUIRE(!(glu && unary) && unary <= SP_UNARY_SILU, "gemm_tiled: activation code %d", glu | (unary << 4));
+    SP_REQUIRE(!(glu && unary) && unary <= SP_UNARY_TANH, "gemm_tiled: activation code %d", glu | (unary << 4));
     g_gate_act = glu ? glu : (unary ? -unary : SP_ACT_SILU);
     if (M == 0) return 0;
     if (shape == 0) {

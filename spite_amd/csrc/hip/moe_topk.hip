@@ -8,7 +8,7 @@
 //     experts' logits z alone (they add up to one; `renorm` has nothing left to do).
 // Outputs expert[t*top + j] and weight[t*top + j] in the order of choice:
 // "virtual tokens" t*top + j that the expert plan (moe_plan with its fan) sorts by expert.
-// moe_combine: out[t] = sum_j weight[t*top + j] * y[t*top + j] (+ extra[t]) in fp32, j in order.
+// moe_combine: out[t] = sum_j weight[t*top + j] * y[t*top + j] (+ extra[t]) in fp32, j in order (no weights: all 1).
 // gated_rows: g[t] = gelu_tanh(a[t]) * table[ids[t]][col0 .. col0 + n): a gate on a per-token row
 // of a table (a second, small embedding that a layer mixes into the stream).
 #include "common.h"
@@ -89,7 +89,7 @@ void moe_combine_kernel(const float* __restrict__ y, const float* __restrict__ w
     if (i >= (size_t)T * d) return;
     const size_t t = i / d, c = i - t * d;
     float acc = 0.f;
-    for (int j = 0; j < top; ++j) acc = fmaf(weight[t * top + j], y[(t * top + j) * d + c], acc);
+    for (int j = 0; j < top; ++j) acc = fmaf(weight ? weight[t * top + j] : 1.0f, y[(t * top + j) * d + c], acc);
     if (extra) acc += extra[i];
     out[i] = acc;
 }

@@ -87,7 +87,7 @@ void act_rows_bf16x8_kernel(bf16x8* __restrict__ x, size_t n8, int act) {
 }
 
 extern "C" int spite_act_rows(void* x, int dtype, size_t n, int act, hipStream_t st) {
-    SP_REQUIRE(act >= SP_UNARY_GELU && act <= SP_UNARY_SILU, "act_rows: activation %d", act);
+    SP_REQUIRE(act >= SP_UNARY_GELU && act <= SP_UNARY_TANH, "act_rows: activation %d", act);
     if (n == 0) return 0;
     if (dtype == SP_BF16 && n % 8 == 0 && ((uintptr_t)x & 15) == 0) {
         const size_t n8 = n / 8;

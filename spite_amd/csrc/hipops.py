@@ -21,7 +21,7 @@ VIS = build.visibility_codes()      # "full", "chunk", "window": name -> code
 GATE_ACTS = {False: 0, None: 0, True: 1, "silu": 1, "gelu_tanh": 2, "relu": 3}
 # an activation of a plain product's own (no gate), as the kernels number them; the bf16 weight-stream and
 # tiled products take it in their epilogue, in the bits above the gate's code
-UNARY_ACTS = {"gelu": 1, "gelu_tanh": 2, "silu": 3}
+UNARY_ACTS = {"gelu": 1, "gelu_tanh": 2, "silu": 3, "tanh": 4}
 
 
 class KernelError(RuntimeError):
@@ -66,15 +66,25 @@ def lib():
             "spite_router_topk": [P, P, P, P, I, I, I, I, I, P],
             "spite_moe_combine": [P, P, P, P, I, I, I, P],
             "spite_gated_rows": [P, I, P, P, I, I, I, P, I, I, P],
-            "spite_qkv_prepare": [P, I, I, P, P, P, F, P, P, P, P, P, P, I, F, P, I, I, I, I, I, I, I, I, I, I, P],
-            "spite_attn_wide": [P, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, I, F, I, I, P, P],
+            "spite_qkv_prepare": [P, I, I, P, P, P, F, P, P, P, P, P, P, I, F, P, I, I, I, I, I, I, I, I, I, I, I, F, I, I, P],
+            "spite_attn_wide": [P, P, P, P, I, I, P, P, P, I, I, I, I, I, I, I, I, I, I, F, I, I, P, P, P],
             "spite_attn_finish": [P, I, P, I, P, P, P, I, I, I, I, I, F, F, F, P],
             "spite_token_shift": [P, P, I, P, P, P, P, P, I, I, I, P],
             "spite_act_rows": [P, I, c_size_t, I, P],
             "spite_scale_rows": [P, c_size_t, F, P],
-            "spite_channel_decay": [P, P, I, I, F, P],
-            "spite_linear_attn_scan": [P, P, P, I, I, I, I, P, P, F, P, I, P, P, I, P, I, I, I, I, I, P],
-            "spite_gated_group_norm": [P, P, I, P, I, P, I, I, I, I, F, I, P],
+            "spite_channel_decay": [P, P, I, I, F, I, P],
+            "spite_linear_attn_scan": [P, P, P, I, I, I, I, P, P, F, P, I, P, P, I, P, I, I, I, I, I, I, P, P, P],
+            "spite_gated_group_norm": [P, P, I, P, I, P, I, I, I, I, F, I, I, P, I, P, I, P],
+            "spite_add_tanh_norm": [P, P, P, P, P, P, P, F, P, P, P, P, I, P, P, I, I, I, P],
+            "spite_hash_rows": [P, P, P, P, P, P, P, I, ctypes.c_longlong, ctypes.c_longlong, ctypes.c_longlong, I, P],
+            "spite_embed_sum": [P, P, P, P, I, P, I, I, I, I, F, P],
+            "spite_causal_conv": [P, I, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+            "spite_shift_mix": [P, I, P, P, P, P, P, P, I, I, I, I, P],
+            "spite_step_decay": [P, I, I, P, P, P, P, I, I, I, P],
+            "spite_softcap_rows": [P, c_size_t, F, P],
+            "spite_axpby_rows": [P, P, P, c_size_t, F, F, P],
+            "spite_concat_rows": [P, P, P, I, I, I, P],
+            "spite_bias_rows": [P, P, P, I, I, P],
         }
         for name, args in sigs.items():
             fn = getattr(l, name)
@@ -708,11 +718,12 @@ def router_topk(logits, bias, expert, weight, top, renorm=False, scoring="sigmoi
 
 
 def moe_combine(y, weight, extra, out, T, top):
-    """out[t] = sum_j weight[t*top + j] * y[t*top + j] (+ extra[t]); all fp32."""
+    """out[t] = sum_j weight[t*top + j] * y[t*top + j] (+ extra[t]); all fp32; ``weight`` None: every weight 1."""
     d = out.shape[-1]
-    if y.numel() < T * top * d or weight.numel() < T * top or out.numel() < T * d or (extra is not None and extra.numel() < T * d):
+    if y.numel() < T * top * d or (weight is not None and weight.numel() < T * top) or out.numel() < T * d \
+            or (extra is not None and extra.numel() < T * d):
         raise KernelError("moe_combine: arrays too small")
-    _check(lib().spite_moe_combine(_ptr(y, "y", torch.float32), _ptr(weight, "weight", torch.float32),
+    _check(lib().spite_moe_combine(_ptr(y, "y", torch.float32), _ptr(weight, "weight", torch.float32, True),
                                    _ptr(extra, "extra", torch.float32, True), _ptr(out, "out", torch.float32),
                                    T, d, int(top), _stream()), "moe_combine")
 
@@ -786,7 +797,8 @@ def attn_latent_mfma(q, kv_pages, out, positions, seq_of_token, block_table, wg,
 # -------------------------------------------------------------------------------------------- keys and values of unequal shape
 def qkv_prepare(qkv, q_out, k_pages, v_pages, positions, slot_map, HQ, GK, GV, D, Vd, page_size, *, bias=None,
                 norm_q=None, norm_k=None, eps=0.0, inv_freq=None, rot=0, inv_freq_v=None, write_kv=True,
-                k_tiled=False, v_tiled=False, stored_dim=None, rot_magnitude=1.0):
+                k_tiled=False, v_tiled=False, stored_dim=None, rot_magnitude=1.0, head_norm=False, q_temperature=None,
+                values_from_keys=False):
     """Between a fused projection and the cache (see attn_wide.hip).  qkv: rows that begin with
     [HQ*D | GK*D | GV*Vd] (further columns are left alone); ``bias`` fp32 over those; ``norm_q`` /
     ``norm_k`` (fp32 [HQ*D], [GK*D]): weights of an RMS norm over the whole q and the whole k part;
@@ -794,10 +806,17 @@ def qkv_prepare(qkv, q_out, k_pages, v_pages, positions, slot_map, HQ, GK, GV, D
     (i, i + rot/2), sine and cosine times ``rot_magnitude``; ``inv_freq_v`` (fp32 [Vd/2]): the values turn in
     pairs (m, m + Vd/2).  q_out
     [T, HQ*Dp]; key pages [pages, GK, page_size, Dp]; value pages [pages, GV, Vd, page_size], with
-    Dp = ``stored_dim`` (default D): queries and keys are stored that wide, zeros behind their D."""
+    Dp = ``stored_dim`` (default D): queries and keys are stored that wide, zeros behind their D.
+    ``head_norm``: ``norm_q`` / ``norm_k`` hold D weights each and every head is normed on its own.
+    ``q_temperature`` = (coef, every): the queries (after their norm) times 1 + coef * ln(floor((p + 1) / every) + 1)
+    at position p.  ``values_from_keys``: the row holds no values, [HQ*D | GK*D] only; the values are the keys as
+    the row holds them, before norm and rotation (GV = GK, Vd = D)."""
     T = qkv.shape[0]
     Dp = int(stored_dim or D)
-    n = (HQ + GK) * D + GV * Vd
+    n = (HQ + GK) * D + (0 if values_from_keys else GV * Vd)
+    if values_from_keys and (GV != GK or Vd != D):
+        raise KernelError("qkv_prepare: values taken from the keys have the keys' heads and width")
+    qt_coef, qt_every = (float(q_temperature[0]), int(q_temperature[1])) if q_temperature else (0.0, 0)
     if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n:
         raise KernelError(f"qkv_prepare: rows {tuple(qkv.shape)} for HQ={HQ} GK={GK} GV={GV} D={D} Vd={Vd}")
     if q_out.numel() < T * HQ * Dp or positions.numel() < T or Dp < D:
@@ -809,7 +828,8 @@ def qkv_prepare(qkv, q_out, k_pages, v_pages, positions, slot_map, HQ, GK, GV, D
                 or k_pages.shape[0] != v_pages.shape[0]:
             raise KernelError(f"qkv_prepare: key pages {tuple(k_pages.shape)}, value pages {tuple(v_pages.shape)} for "
                               f"GK={GK} GV={GV} page={page_size} D={D} Vd={Vd}")
-    for name, t, size in (("bias", bias, n), ("norm_q", norm_q, HQ * D), ("norm_k", norm_k, GK * D),
+    for name, t, size in (("bias", bias, n), ("norm_q", norm_q, D if head_norm else HQ * D),
+                          ("norm_k", norm_k, D if head_norm else GK * D),
                           ("inv_freq", inv_freq, rot // 2), ("inv_freq_v", inv_freq_v, Vd // 2)):
         if t is not None and t.numel() != size:
             raise KernelError(f"qkv_prepare: {name} of {t.numel()} values, expected {size}")
@@ -823,15 +843,17 @@ def qkv_prepare(qkv, q_out, k_pages, v_pages, positions, slot_map, HQ, GK, GV, D
         _ptr(positions, "positions", torch.int32), _ptr(slot_map, "slot_map", torch.int32) if write_kv else None,
         _ptr(inv_freq, "inv_freq", torch.float32, True), int(rot), float(rot_magnitude),
         _ptr(inv_freq_v, "inv_freq_v", torch.float32, True),
-        T, HQ, GK, GV, D, Vd, page_size, int(bool(k_tiled)), int(bool(v_tiled)), Dp, _stream()), "qkv_prepare")
+        T, HQ, GK, GV, D, Vd, page_size, int(bool(k_tiled)), int(bool(v_tiled)), Dp, int(bool(head_norm)), qt_coef, qt_every,
+        int(bool(values_from_keys)), _stream()), "qkv_prepare")
 
 
 def attn_wide(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T, HQ, GK, GV, D, Vd, page_size, vis, span,
-              scale, k_tiled=False, v_tiled=False, sinks=None):
+              scale, k_tiled=False, v_tiled=False, sinks=None, slopes=None):
     """Attention over the paged cache with keys of D and values of Vd elements, HQ query heads over
     GK key heads over GV value heads (query head h: key head h // (HQ/GK), value head of that % GV);
     any mix of portions and single tokens.  q [T, HQ*D]; out [T, HQ*Vd] in q's dtype or fp32.
-    ``sinks`` (fp32 [HQ] or None): one more term exp(sinks[h]) in every softmax's denominator."""
+    ``sinks`` (fp32 [HQ] or None): one more term exp(sinks[h]) in every softmax's denominator.
+    ``slopes`` (fp32 [HQ] or None): slopes[h] * (key position - query position) is added to the scaled score."""
     if sinks is not None and sinks.numel() != HQ:
         raise KernelError(f"attention: {sinks.numel()} sinks for {HQ} query heads")
     if q.numel() < T * HQ * D or out.numel() < T * HQ * Vd:
@@ -848,7 +870,7 @@ def attn_wide(q, k_pages, v_pages, out, positions, seq_of_token, block_table, T,
         dtype_code(out.dtype), _ptr(positions, "positions", torch.int32), _ptr(seq_of_token, "seq_of_token", torch.int32),
         _ptr(block_table, "block_table", torch.int32), block_table.shape[1], T, HQ, GK, GV, D, Vd, page_size,
         VIS[vis], int(span or 0), float(scale), int(bool(k_tiled)), int(bool(v_tiled)),
-        _ptr(sinks, "sinks", torch.float32, True), _stream()), "attention")
+        _ptr(sinks, "sinks", torch.float32, True), _slopes(slopes, HQ), _stream()), "attention")
 
 
 def attn_finish(a, out, positions, H, Vd, *, maps=1, lam=0.0, eps=0.0, post=1.0, inv_freq_v=None, gate=None):
@@ -901,15 +923,21 @@ def scale_rows(x, c: float):
 
 
 # -------------------------------------------------------------------------------------------- linear attention
-def channel_decay(z, bias, tau: float):
-    """z[t, c] = sigmoid(z[t, c] + bias[c]) ** (1 / tau) in place; z fp32 [T, n], bias fp32 [n] or None."""
+DECAY_FORMS = {"sigmoid_root": 0, "exp_exp": 1}
+
+
+def channel_decay(z, bias, tau: float = 1.0, form: str = "sigmoid_root"):
+    """z[t, c] = sigmoid(z[t, c] + bias[c]) ** (1 / tau) in place (``form`` ``sigmoid_root``), or
+    exp(-exp(z[t, c] + bias[c])) (``exp_exp``); z fp32 [T, n], bias fp32 [n] or None."""
+    if form not in DECAY_FORMS:
+        raise KernelError(f"channel_decay: form {form!r} (known: {sorted(DECAY_FORMS)})")
     T, n = z.shape
     if bias is not None and bias.numel() != n:
         raise KernelError(f"channel_decay: bias of {bias.numel()} for rows of {n}")
     if not tau > 0:
         raise KernelError(f"channel_decay: tau = {tau}")
     _check(lib().spite_channel_decay(_ptr(z, "z", torch.float32), _ptr(bias, "bias", torch.float32, True), T, n,
-                                     1.0 / float(tau), _stream()), "channel_decay")
+                                     1.0 / float(tau), DECAY_FORMS[form], _stream()), "channel_decay")
 
 
 def _rows_view(t, name, width, T):
@@ -920,18 +948,24 @@ def _rows_view(t, name, width, T):
 
 
 def linear_attn_scan(q, k, v, out, state, cu_seqlens, seq_slots, n_seqs, H, D, V, *, decay=None, head_decay=None,
-                     q_scale=1.0, keep=True, longest=0):
+                     q_scale=1.0, keep=True, longest=0, qk_heads=None, v_scale=None, bonus=None):
     """The recurrence S = diag(a) S + k v^T, o = S^T q token by token for every entry of the step (see
     linear_attn.hip).  q, k [T, H*D] and v [T, H*V]: views of the run's dtype whose rows may lie apart;
     ``decay`` fp32 [T, H*D] (a number per key channel and token) or ``head_decay`` fp32 [H]; ``state`` fp32
     [slots, H, D, V], read at the entry's slot and, with ``keep``, left as the entry's last token leaves it;
     out fp32 [T, H*V].  ``longest``: the most tokens an entry has, if the caller knows (1 picks the kernel made
-    for single tokens; the results are the same bits either way)."""
+    for single tokens; the results are the same bits either way).  ``qk_heads`` < H: q and k have that many heads
+    ([T, qk_heads*D]) and head h reads head h // (H / qk_heads) of them.  ``v_scale`` fp32 [T, H]: a factor on a
+    head's value row as it enters the state.  ``bonus`` fp32 [H, D] (with ``decay``): the result is read before the
+    token enters the state, o = (S + diag(bonus) k v^T)^T q."""
     T = out.shape[0]
+    Hq = int(qk_heads or H)
+    if H % Hq:
+        raise KernelError(f"linear_attn_scan: {H} heads over {Hq} heads of q and k")
     if q.dtype != k.dtype or q.dtype != v.dtype:
         raise KernelError("linear_attn_scan: q, k and v of one dtype")
-    pq, ldq = _rows_view(q, "q", H * D, T)
-    pk, ldk = _rows_view(k, "k", H * D, T)
+    pq, ldq = _rows_view(q, "q", Hq * D, T)
+    pk, ldk = _rows_view(k, "k", Hq * D, T)
     pv, ldv = _rows_view(v, "v", H * V, T)
     if out.numel() < T * H * V or tuple(state.shape[1:]) != (H, D, V):
         raise KernelError(f"linear_attn_scan: out {tuple(out.shape)}, state {tuple(state.shape)} for H={H} D={D} V={V}")
@@ -941,21 +975,34 @@ def linear_attn_scan(q, k, v, out, state, cu_seqlens, seq_slots, n_seqs, H, D, V
         raise KernelError(f"linear_attn_scan: {head_decay.numel()} decays for {H} heads")
     if cu_seqlens.numel() < n_seqs + 1 or seq_slots.numel() < n_seqs:
         raise KernelError("linear_attn_scan: metadata too small")
+    if v_scale is not None and v_scale.numel() < T * H:
+        raise KernelError("linear_attn_scan: v_scale too small")
+    if bonus is not None and (bonus.numel() != H * D or decay is None):
+        raise KernelError(f"linear_attn_scan: a bonus of {H} x {D} numbers, with a decay per channel")
     _check(lib().spite_linear_attn_scan(
         pq, pk, pv, ldq, ldk, ldv, dtype_code(q.dtype), _ptr(decay, "decay", torch.float32, True),
         _ptr(head_decay, "head_decay", torch.float32, True), float(q_scale), _ptr(state, "state", torch.float32),
         state.shape[0], _ptr(cu_seqlens, "cu_seqlens", torch.int32), _ptr(seq_slots, "seq_slots", torch.int32), int(n_seqs),
-        _ptr(out, "out", torch.float32), H, D, V, int(bool(keep)), int(longest), _stream()), "linear_attn_scan")
+        _ptr(out, "out", torch.float32), H, D, V, int(bool(keep)), int(longest), Hq,
+        _ptr(v_scale, "v_scale", torch.float32, True), _ptr(bonus, "bonus", torch.float32, True), _stream()), "linear_attn_scan")
 
 
 NORM_GATES = {None: 0, "silu": 1, "sigmoid": 2}
 
 
-def gated_group_norm(o, weight, y, group, eps, gate=None, act=None):
+def gated_group_norm(o, weight, y, group, eps, gate=None, act=None, gate_first=False, skip=None, skip_weight=None,
+                     skip_group=0):
     """y = rmsnorm(o over groups of ``group`` elements) * weight * act(gate).  o fp32 [T, n]; weight fp32
     of ``group`` elements (shared by the groups) or of n; gate a [T, n] view in y's dtype (rows may lie
-    apart) with ``act`` silu or sigmoid, or None; y [T, n]."""
+    apart) with ``act`` silu or sigmoid, or None; y [T, n].  ``gate_first``: y = rmsnorm(o * act(gate)) * weight.
+    ``skip`` (a [T, n] view in y's dtype) with ``skip_weight`` fp32 [n / skip_group]: o + skip_weight[head] * skip
+    stands for o."""
     T, n = o.shape
+    ps, lds = (None, 0)
+    if skip is not None:
+        if skip.dtype != y.dtype or skip_weight is None or skip_group <= 0 or n % skip_group or skip_weight.numel() != n // skip_group:
+            raise KernelError("gated_group_norm: the skip rows have the output's dtype and one weight a head")
+        ps, lds = _rows_view(skip, "skip", n, T)
     if act not in NORM_GATES or (act is None) != (gate is None):
         raise KernelError(f"gated_group_norm: gate activation {act!r} (known: silu, sigmoid) with a gate, or neither")
     pg, ldg = (None, 0)
@@ -967,4 +1014,138 @@ def gated_group_norm(o, weight, y, group, eps, gate=None, act=None):
         raise KernelError("gated_group_norm: output too small")
     _check(lib().spite_gated_group_norm(_ptr(o, "o", torch.float32), pg, ldg, _ptr(weight, "weight", torch.float32),
                                         weight.numel(), _ptr(y, "y"), dtype_code(y.dtype), T, n, int(group), float(eps),
-                                        NORM_GATES[act], _stream()), "gated_group_norm")
+                                        NORM_GATES[act], int(bool(gate_first)), ps, lds,
+                                        _ptr(skip_weight, "skip_weight", torch.float32, True), int(skip_group), _stream()),
+           "gated_group_norm")
+
+
+# -------------------------------------------------------------------------------------------- parts around the stream
+def add_tanh_norm(h, w, b, alpha, out=None, out32=None, d1=None, d2=None, rows=None, n_rows=None, write_h=True, normed=None):
+    """h (fp32 [T,d]) += d1 + d2 + mult * (tanh(an * yn) * wn + bn) with ``normed`` = (yn, wn, bn, an, mult); then
+    out[i] (and out32[i]) = tanh(alpha * h[r]) * w + b, r = rows[i] or i.  ``w`` None: out is the stream itself in
+    out's dtype.  alpha and an are fp32 tensors of one element."""
+    T, d = h.shape
+    n = int(n_rows if n_rows is not None else (rows.numel() if rows is not None else T))
+    for name, t in (("d1", d1), ("d2", d2)):
+        if t is not None and (t.numel() < T * d or t.dtype != torch.float32):
+            raise KernelError(f"add_tanh_norm: increment {name} too small or not fp32")
+    if w is not None and (w.numel() != d or b is None or b.numel() != d or alpha is None or alpha.numel() != 1):
+        raise KernelError(f"add_tanh_norm: weight, bias of {d} elements and one alpha")
+    yn = wn = bn = an = None
+    mult = 0.0
+    if normed is not None:
+        yn, wn, bn, an, mult = normed
+        if yn.numel() < T * d or wn.numel() != d or bn.numel() != d or an.numel() != 1:
+            raise KernelError("add_tanh_norm: the normed increment's sizes")
+    if rows is not None and (write_h or rows.numel() < n):
+        raise KernelError("add_tanh_norm: gathered rows do not write the stream")
+    for name, t in (("out", out), ("out32", out32)):
+        if t is not None and t.numel() < n * d:
+            raise KernelError(f"add_tanh_norm: {name} too small")
+    f = torch.float32
+    _check(lib().spite_add_tanh_norm(
+        _ptr(h, "h", f), _ptr(d1, "d1", f, True), _ptr(d2, "d2", f, True), _ptr(yn, "yn", f, True), _ptr(wn, "wn", f, True),
+        _ptr(bn, "bn", f, True), _ptr(an, "an", f, True), float(mult), _ptr(w, "w", f, True), _ptr(b, "b", f, True),
+        _ptr(alpha, "alpha", f, True), _ptr(out, "out", None, True), dtype_code(out.dtype) if out is not None else F32,
+        _ptr(out32, "out32", f, True), _ptr(rows, "rows", torch.int32, True), n, d, int(bool(write_h)), _stream()), "add_tanh_norm")
+
+
+def hash_rows(ids, positions, seq_of_token, cu_seqlens, seq_slots, state, rows, mul_prev, mul_cur, buckets, keep=True):
+    """rows[t] = (previous token * mul_prev + token * mul_cur) mod buckets, ``buckets`` itself at position 0.  The
+    previous token of an entry's first token is state[slot] (int32 [slots]), which then takes the entry's last token."""
+    T = rows.numel()
+    if ids.numel() < T or positions.numel() < T or seq_of_token.numel() < T or state.dim() != 1:
+        raise KernelError("hash_rows: arrays too small")
+    i32 = torch.int32
+    _check(lib().spite_hash_rows(_ptr(ids, "ids", i32), _ptr(positions, "positions", i32), _ptr(seq_of_token, "seq_of_token", i32),
+                                 _ptr(cu_seqlens, "cu_seqlens", i32), _ptr(seq_slots, "seq_slots", i32), _ptr(state, "state", i32),
+                                 _ptr(rows, "rows", i32), T, int(mul_prev), int(mul_cur), int(buckets), int(bool(keep)), _stream()),
+           "hash_rows")
+
+
+def embed_sum(ids, table, rows2, table2, h, scale=1.0):
+    """h[t] = table[ids[t]] * scale + table2[rows2[t]] as fp32."""
+    T, d = h.shape
+    if table.shape[1] != d or table2.shape[1] != d or table.dtype != table2.dtype or ids.numel() < T or rows2.numel() < T:
+        raise KernelError("embed_sum: tables of the stream's width and one dtype")
+    _check(lib().spite_embed_sum(_ptr(ids, "ids", torch.int32), _ptr(table, "table"), _ptr(rows2, "rows2", torch.int32),
+                                 _ptr(table2, "table2"), dtype_code(table.dtype), _ptr(h, "h", torch.float32), T, d,
+                                 table.shape[0], table2.shape[0], float(scale), _stream()), "embed_sum")
+
+
+CONV_ACTS = {None: 0, "silu": 1}
+
+
+def causal_conv(x, w, y, state, seq_of_token, cu_seqlens, seq_slots, bias=None, act=None, keep=True):
+    """y[t, c] = act(bias[c] + sum_j w[c, j] * x[t - taps + 1 + j, c]) within a request; the inputs before an entry's
+    first token come from state (fp32 [slots, taps-1, C]), which then holds the request's last taps - 1 inputs.  x and y:
+    [T, C] views of one dtype whose rows may lie apart; w fp32 [C, taps]."""
+    T = y.shape[0]
+    C, taps = w.shape
+    px, ldx = _rows_view(x, "x", C, T)
+    py, ldy = _rows_view(y, "y", C, T)
+    if x.dtype != y.dtype or act not in CONV_ACTS or (bias is not None and bias.numel() != C):
+        raise KernelError("causal_conv: x and y of one dtype, activation silu or none, a bias per channel")
+    if taps > 1 and (state is None or tuple(state.shape[1:]) != (taps - 1, C)):
+        raise KernelError(f"causal_conv: state {None if state is None else tuple(state.shape)} for {taps} taps on {C} channels")
+    if seq_of_token.numel() < T:
+        raise KernelError("causal_conv: metadata too small")
+    _check(lib().spite_causal_conv(px, ldx, dtype_code(x.dtype), _ptr(w, "w", torch.float32), _ptr(bias, "bias", torch.float32, True),
+                                   _ptr(state, "state", torch.float32, True), _ptr(seq_of_token, "seq_of_token", torch.int32),
+                                   _ptr(cu_seqlens, "cu_seqlens", torch.int32), _ptr(seq_slots, "seq_slots", torch.int32),
+                                   py, ldy, dtype_code(y.dtype), T, C, taps, CONV_ACTS[act], int(bool(keep)), _stream()), "causal_conv")
+
+
+def shift_mix(x, mu, state, y, seq_of_token, cu_seqlens, seq_slots, keep=True):
+    """y[s, t] = x[t] + (x[t-1] - x[t]) * mu[s] within a request, s over the rows of mu (fp32 [n, d]); the row before
+    an entry's first token is state[slot] (fp32 [slots, d]), which then takes the entry's last row.  x [T, d], y [n, T, d]."""
+    T, d = x.shape
+    n = mu.shape[0]
+    if tuple(y.shape) != (n, T, d) or y.dtype != x.dtype or mu.shape[1] != d or tuple(state.shape[1:]) != (d,) or seq_of_token.numel() < T:
+        raise KernelError(f"shift_mix: x {tuple(x.shape)}, mu {tuple(mu.shape)}, y {tuple(y.shape)}, state {tuple(state.shape)}")
+    _check(lib().spite_shift_mix(_ptr(x, "x"), dtype_code(x.dtype), _ptr(mu, "mu", torch.float32), _ptr(state, "state", torch.float32),
+                                 _ptr(y, "y"), _ptr(seq_of_token, "seq_of_token", torch.int32), _ptr(cu_seqlens, "cu_seqlens", torch.int32),
+                                 _ptr(seq_slots, "seq_slots", torch.int32), T, d, n, int(bool(keep)), _stream()), "shift_mix")
+
+
+def step_decay(raw, dt_bias, a_log, dt, decay, H, N):
+    """dt[t, h] = softplus(raw[t, h] + dt_bias[h]); decay[t, h*N + n] = exp(-exp(a_log[h]) * dt[t, h]).  raw: a [T, H]
+    view whose rows may lie apart; dt fp32 [T, H]; decay fp32 [T, H*N]."""
+    T = dt.shape[0]
+    pr, ld = _rows_view(raw, "raw", H, T)
+    if dt.numel() < T * H or decay.numel() < T * H * N or dt_bias.numel() != H or a_log.numel() != H:
+        raise KernelError("step_decay: arrays too small")
+    _check(lib().spite_step_decay(pr, ld, dtype_code(raw.dtype), _ptr(dt_bias, "dt_bias", torch.float32), _ptr(a_log, "a_log", torch.float32),
+                                  _ptr(dt, "dt", torch.float32), _ptr(decay, "decay", torch.float32), T, H, N, _stream()), "step_decay")
+
+
+def softcap_rows(x, cap: float):
+    """x = cap * tanh(x / cap) in place; x fp32."""
+    _check(lib().spite_softcap_rows(_ptr(x, "x", torch.float32), x.numel(), float(cap), _stream()), "softcap_rows")
+
+
+def axpby_rows(x, y, out, a: float, b: float):
+    """out = a * x + b * y; all fp32 of one size (out may be x or y)."""
+    if x.numel() != y.numel() or out.numel() != x.numel():
+        raise KernelError("axpby_rows: sizes differ")
+    f = torch.float32
+    _check(lib().spite_axpby_rows(_ptr(x, "x", f), _ptr(y, "y", f), _ptr(out, "out", f), x.numel(), float(a), float(b), _stream()),
+           "axpby_rows")
+
+
+def concat_rows(a, b, out):
+    """out[t] = [a[t] | b[t]] in out's dtype; a, b fp32 [T, d], out [T, 2d]."""
+    T, d = a.shape
+    if tuple(b.shape) != (T, d) or tuple(out.shape) != (T, 2 * d):
+        raise KernelError("concat_rows: shapes")
+    f = torch.float32
+    _check(lib().spite_concat_rows(_ptr(a, "a", f), _ptr(b, "b", f), _ptr(out, "out"), dtype_code(out.dtype), T, d, _stream()), "concat_rows")
+
+
+def bias_rows(y, v, out):
+    """out[t] = y[t] + v; y, out fp32 [T, d], v fp32 [d]."""
+    T, d = y.shape
+    if v.numel() != d or out.numel() < T * d:
+        raise KernelError("bias_rows: shapes")
+    f = torch.float32
+    _check(lib().spite_bias_rows(_ptr(y, "y", f), _ptr(v, "v", f), _ptr(out, "out", f), T, d, _stream()), "bias_rows")

@@ -33,6 +33,12 @@ class Model:
             if wanted != given and not (len(wanted) == 1 and given == {""}):
                 raise ValueError(f"layer call {i}: block {call.block} has the caches {sorted(wanted)}, the call names {sorted(given)}")
         writers = {}
+        self.embedding_cache = None
+        if self.embedding.state_need() is not None:
+            if spec.embedding_cache is None:
+                raise ValueError(f"the embedding {self.embedding_spec.kind!r} keeps a state per request: the spec must give it a cache id")
+            self.embedding_cache = int(spec.embedding_cache)
+            writers[self.embedding_cache] = -1
         for i, call in enumerate(spec.order):
             if call.write:
                 for cid in call.cache_ids().values():
@@ -76,8 +82,13 @@ class Model:
     def cache_needs(self) -> List[Optional[CacheNeed]]:
         """What every cache id asks for: what the block of the call that writes it says."""
         n = max((cid for c in self.spec.order for cid in c.cache_ids().values()), default=-1) + 1
+        if self.embedding_cache is not None:
+            n = max(n, self.embedding_cache + 1)
         needs: List[Optional[CacheNeed]] = [None] * n
         for cid, i in self._writers.items():
+            if i < 0:                                  # the embedding's state
+                needs[cid] = CacheNeed(state=self.embedding.state_need())
+                continue
             call = self.spec.order[i]
             of_block = self.blocks[call.block].cache_needs()
             for name, c in call.cache_ids().items():
@@ -120,11 +131,17 @@ class Model:
                 state["h"] = step_ws.take((ctx.T, d), torch.float32)
                 state["pending"] = ()
                 ctx.ws = arenas[0]
-                self.embedding.forward(ctx.token_ids, state["h"], ctx)
+                estate = cache.states.get(self.embedding_cache) if self.embedding_cache is not None else None
+                self.embedding.forward(ctx.token_ids, state["h"], ctx, state=estate)
+                if self.spec.keep_embedding:
+                    # a copy for the blocks that read the embedding's result later in the step (the norms change h in place)
+                    state["h0"] = step_ws.take((ctx.T, d), torch.float32)
+                    state["h0"].copy_(state["h"])
             elif kind == "stage":
                 ctx.ws = arenas[i % 2]
                 if stage[0] == 0:
                     ctx.ws.reset()
+                ctx.extras["call"] = self.spec.order[i]
                 stage[1](state, ctx, meta.layer_cache(cache, self.spec.order[i]))
             else:
                 ctx.ws = arenas[n % 2]

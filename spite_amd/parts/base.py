@@ -85,6 +85,8 @@ class LayerCall:
     block: int                   # index into ModelSpec.blocks
     cache: Any                   # cache id; the call with write=True fills it.  A block with several caches
     write: bool = True           # (``Block.cache_needs``) names them all: {the block's name of a cache: cache id}
+    arg: Any = None              # what this call of the block differs by from its other calls (the number of a pass);
+                                 # the block finds the call under ``ctx.extras["call"]``
 
     def cache_ids(self) -> Dict[str, int]:
         """{the block's name of a cache: cache id}; a call with one id serves a block with one cache."""
@@ -107,6 +109,8 @@ class ModelSpec:
     ignore_prefixes: Tuple[str, ...] = ()   # tensors of the checkpoint that belong to no part of this model
     embedding: Optional[PartSpec] = None    # other kinds of the two ends than the shorthands above name
     head: Optional[PartSpec] = None
+    embedding_cache: Optional[int] = None   # cache id of the embedding's per-request state, if it keeps one
+    keep_embedding: bool = False            # blocks read the embedding's result later in the step (``state["h0"]``)
 
 
 class Part:
@@ -169,6 +173,12 @@ class Mixer(Part):
     def cache_need(self) -> CacheNeed:
         return CacheNeed()
 
+    def cache_needs(self) -> Dict[str, CacheNeed]:
+        """A mixer that keeps more than pages and one state tensor names each of its caches (two mixers side by
+        side; a recurrent state beside the last inputs of a convolution); its block's layer calls give every name a
+        cache id and ``forward`` gets a dict of ``LayerCache`` by those names.  Default: the one ``cache_need``."""
+        return {"": self.cache_need()}
+
     def forward(self, x, ctx, cache):
         """x [T,d] in the run's dtype -> fp32 [T,d], the residual's increment, taken from
         ``ctx.ws`` (it must stay valid until the next layer call has consumed it)."""
@@ -216,8 +226,14 @@ class Embedding(Part):
     #: the table [V, d] after loading, for a head that is tied to it (None if there is none)
     table = None
 
-    def forward(self, token_ids, h, ctx) -> None:
-        """h (fp32 [T,d]) = the residual stream's first value for the step's token ids (int32 [T])."""
+    def state_need(self) -> Optional[StateNeed]:
+        """What the embedding remembers of a request between steps (its last token, say), or None.  The model
+        spec gives it a cache id (``ModelSpec.embedding_cache``) and ``forward`` gets the state tensor."""
+        return None
+
+    def forward(self, token_ids, h, ctx, state=None) -> None:
+        """h (fp32 [T,d]) = the residual stream's first value for the step's token ids (int32 [T]); ``state``: the
+        ``[max_requests, ...]`` tensor that ``state_need`` asked for."""
         raise NotImplementedError
 
 
@@ -242,18 +258,44 @@ class NormedIncrement:
     def as_arg(self):
         return (self.y, self.weight, self.mult, self.eps)
 
+    def add_to(self, h) -> None:
+        """Adds the increment to the stream in a pass of its own (where no norm takes it on its way)."""
+        from ..csrc import hipops
+        hipops.add_rmsnorm(h, None, self.eps, normed=self.as_arg())
+
+
+@dataclass
+class TanhIncrement:
+    """An increment that passes a tanh norm first: h += mult * (tanh(alpha * y) * weight + bias).  The tanh norm's
+    kernel takes one beside its plain increments."""
+    y: torch.Tensor              # fp32 [T, d]
+    weight: torch.Tensor         # fp32 [d]
+    bias: torch.Tensor           # fp32 [d]
+    alpha: torch.Tensor          # fp32, one element
+    mult: float
+
+    def as_arg(self):
+        return (self.y, self.weight, self.bias, self.alpha, self.mult)
+
+    def add_to(self, h) -> None:
+        from ..csrc import hipops
+        hipops.add_tanh_norm(h, None, None, None, normed=self.as_arg())
+
+
+#: increments that pass a norm of their own on their way into the stream
+NORMED_INCREMENTS = (NormedIncrement, TanhIncrement)
+
 
 def two_increments(h, pending):
     """A norm adds up to two increments to the residual stream itself; what ``pending`` holds beyond
     two (a feed-forward with three or more results a token, each written by a grouped product
     to rows of its own) is added to ``h`` here first, in order.  Returns the two for the norm.
     A ``NormedIncrement`` left by a block whose successor does not take it itself is added here."""
-    if any(isinstance(p, NormedIncrement) for p in pending):
-        from ..csrc import hipops
+    if any(isinstance(p, NORMED_INCREMENTS) for p in pending):
         for p in pending:
-            if isinstance(p, NormedIncrement):
-                hipops.add_rmsnorm(h, None, p.eps, normed=p.as_arg())
-        pending = tuple(p for p in pending if not isinstance(p, NormedIncrement))
+            if isinstance(p, NORMED_INCREMENTS):
+                p.add_to(h)
+        pending = tuple(p for p in pending if not isinstance(p, NORMED_INCREMENTS))
     if len(pending) > 2:
         from ..csrc import hipops
         for d in pending[2:]:

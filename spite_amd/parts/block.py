@@ -6,7 +6,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import Block, NormedIncrement, register, build as build_part, two_increments
+from .base import Block, NormedIncrement, NORMED_INCREMENTS, register, build as build_part, two_increments
 
 
 @register("block", "prenorm")
@@ -71,7 +71,8 @@ class SandwichBlock(Block):
     then, if the layer has one, a side input from the step's tokens (``spec.extra["side"]``).  The
     feed-forward may be missing.  ``spec.extra``: ``norm1b``, ``norm2b`` (PartSpecs), ``residual_mult``.
     Every addition is folded into the norm kernel that next reads the stream (a normed increment
-    beside the plain ones); the last one is handed to the next block."""
+    beside the plain ones); the last one is handed to the next block.  The norms are of any kind that
+    offers ``as_increment`` (RMS, tanh).  A mixer with several caches (``Mixer.cache_needs``) gets them by name."""
     graph_safe = True
 
     def __init__(self, env, spec):
@@ -97,6 +98,9 @@ class SandwichBlock(Block):
         self.graph_safe = all(part.graph_safe for _, part, _ in self.children)
         self.step_arrays = tuple(sorted({a for _, part, _ in self.children for a in part.step_arrays}))
 
+    def cache_needs(self):
+        return self.mixer.cache_needs()
+
     def forward(self, h, pending, ctx, cache):
         state = {"h": h, "pending": pending}
         for _, stage in self.stages():
@@ -109,16 +113,18 @@ class SandwichBlock(Block):
                 (rest, self._stage_rest)]
 
     @staticmethod
-    def _split(h, pending):
-        """(d1, d2, one normed increment or None) of what is still to be added to h."""
-        normed = [p for p in pending if isinstance(p, NormedIncrement)]
+    def _split(h, pending, norm=None):
+        """(d1, d2, one normed increment or None) of what is still to be added to h; the normed increment is one
+        that ``norm`` (default: an RMS norm) adds in its own pass."""
+        takes = norm.takes if norm is not None and hasattr(norm, "takes") else (lambda p: isinstance(p, NormedIncrement))
+        normed = [p for p in pending if isinstance(p, NORMED_INCREMENTS) and takes(p)]
         last = normed.pop() if normed else None
         d1, d2 = two_increments(h, tuple(p for p in pending if p is not last))
         return d1, d2, (last.as_arg() if last is not None else None)
 
     def _stage_norm1(self, state, ctx, cache):
         h = state["h"]
-        d1, d2, normed = self._split(h, state["pending"])
+        d1, d2, normed = self._split(h, state["pending"], self.norm1)
         n = ctx.ws.take(tuple(h.shape), self.env.dtype)
         self.norm1.forward(h, n, d1=d1, d2=d2, normed=normed)
         state["normed"] = n
@@ -273,3 +279,82 @@ class ParallelBlock(Block):
         if self.side is not None:
             pend = tuple(self.side.forward(state["h"], pend, ctx))
         state["pending"] = pend
+
+
+@register("block", "reentry")
+class ReentryBlock(Block):
+    """No layer, but what stands before a run of layers that is walked several times with the same weights: the
+    stream is mixed with the embedding's result again and a vector of the pass is added,
+
+        x <- W [x ; x0] + step[pass],
+
+    W ``[d, 2d]`` (the stream's columns first), x0 what the embedding left at the start of the step
+    (``ModelSpec.keep_embedding``), ``step`` ``[passes, d]``.  ``spec.extra``: ``width``, ``passes``, ``names`` (the
+    two tensors); the number of the pass is the layer call's ``arg``.  It has no cache."""
+    graph_safe = True
+
+    def __init__(self, env, spec):
+        from .base import ParamSpec, PartSpec
+        from .norm import TanhNorm  # noqa: F401  (the increments' kinds are registered)
+        self.env = env
+        ex = spec.extra
+        self.d, self.passes = int(ex["width"]), int(ex["passes"])
+        self.mixer = None
+        self.w = self.step = None
+        self._inner = _ReentryTensors(self)
+        self.children = (("reentry", self._inner, PartSpec("reentry", {}, dict(ex["names"]))),)
+        self.step_arrays = ()
+
+    def cache_needs(self):
+        return {}
+
+    def forward(self, h, pending, ctx, cache):
+        from ..csrc import hipops
+        from .linear import linear
+        T, d, ws = h.shape[0], self.d, ctx.ws
+        h0 = ctx.extras.get("h0")
+        if h0 is None:
+            raise ValueError("reentry: the model spec does not keep the embedding's result (keep_embedding)")
+        d1, d2 = two_increments(h, pending)                 # everything still on its way joins the stream first
+        if d1 is not None:
+            hipops.add_into(h, d1[:T])
+        if d2 is not None:
+            hipops.add_into(h, d2[:T])
+        both = ws.take((T, 2 * d), self.env.dtype)
+        hipops.concat_rows(h, h0, both)
+        y = ws.take((T, d), torch.float32)
+        linear(both, self.w, y, ws=ws)
+        which = int(ctx.extras["call"].arg or 0)
+        if not 0 <= which < self.passes:
+            raise ValueError(f"reentry: pass {which} of {self.passes}")
+        hipops.bias_rows(y, self.step[which], h)
+        return ()
+
+    def stages(self):
+        def whole(state, ctx, cache):
+            ctx.extras["h0"] = state.get("h0")
+            state["pending"] = self.forward(state["h"], state["pending"], ctx, cache)
+        return [(True, whole)]
+
+
+class _ReentryTensors:
+    """The tensors of a ``reentry`` block, as the loader sees a part."""
+    graph_safe = True
+    step_arrays = ()
+
+    def __init__(self, block):
+        self.block = block
+
+    def params(self):
+        from .base import ParamSpec
+        b = self.block
+        return {"mix": ParamSpec((b.d, 2 * b.d)), "step": ParamSpec((b.passes, b.d), kind="vector", init="normal")}
+
+    def load(self, t):
+        from .linear import Weight
+        b = self.block
+        b.w = Weight(t["mix"])
+        b.step = t["step"].float().contiguous()
+
+    def slow_paths(self, page_size):
+        return self.block.w.slow_reason("reentry matrix") if self.block.w is not None else []

@@ -21,6 +21,9 @@ expert of its own width may run for every token.  The choices of a step are ``to
 token; the expert plan sorts them by expert, the grouped products walk that list, every entry
 gets an output row of its own and a last kernel forms the weighted sum per token.
 
+With ``weight_input`` the weight multiplies the expert's input instead (the grouped product scales the rows it
+reads) and the outputs are summed as they are.
+
 ``moe_topk_softmax``: the same part with the other way of scoring: the ``top_k`` experts with the largest
 logits are taken and their weights are the softmax over the taken logits alone; no bias.
 """
@@ -216,9 +219,11 @@ class MoeTopKSigmoid(FeedForward):
     wants_f32_input = True
 
     def __init__(self, env, hidden_size, intermediate_size, n_experts, top_k, shared_intermediate_size=None,
-                 score_bias=True, renormalize=False, activation="silu", scoring="sigmoid"):
+                 score_bias=True, renormalize=False, activation="silu", scoring="sigmoid", weight_input=False):
         """``scoring``: ``sigmoid`` (the choice by sigmoid(z) + bias, weights sigmoid(z)) or ``softmax_taken`` (the
-        choice by z + bias, weights the softmax over the taken experts' z)."""
+        choice by z + bias, weights the softmax over the taken experts' z).  ``weight_input``: the weight multiplies
+        the expert's input instead of its output: the result is the sum of expert(w * x)."""
+        self.weight_input = bool(weight_input)
         if scoring not in hipops.ROUTER_SCORING:
             raise ValueError(f"moe: scoring {scoring!r} (known: {sorted(hipops.ROUTER_SCORING)})")
         self.scoring = scoring
@@ -286,14 +291,15 @@ class MoeTopKSigmoid(FeedForward):
         hipops.router_topk(logits, bias, expert, weight, k, renorm=self.renormalize, scoring=self.scoring)
         if trace is not None:                         # a testing aid: which experts each token took, [T, top_k]
             trace.setdefault("moe_experts", []).append(expert.view(T, k).clone())
+        # (``unused``: the entries' weights in the order of the slots; a product reads it only with ``weight_input``)
         src, dst, unused = ws.take((n,), torch.int32), ws.take((n,), torch.int32), ws.take((n,), torch.float32)
         offsets = ws.take((E + 1,), torch.int32)
         hipops.moe_plan(expert, weight, src, unused, dst, offsets, n, E, False, fan=k)
         live = min(n, E)
         # slot s (entries sorted by expert) reads token src[s] and writes the entry's own row dst[s]
         act = ws.take((n, F), x.dtype)
-        linear(x, self.w_gate_up, act, glu=self.activation, offsets=offsets, n_groups=E, a_rows=src, rows=n, max_rows=T,
-               live_groups=live, ws=ws)
+        linear(x, self.w_gate_up, act, glu=self.activation, offsets=offsets, n_groups=E, a_rows=src,
+               a_scale=unused if self.weight_input else None, rows=n, max_rows=T, live_groups=live, ws=ws)
         y = ws.take((n, d), torch.float32)
         linear(act, self.w_down, y, offsets=offsets, n_groups=E, y_rows=dst, rows=n, max_rows=T, live_groups=live, ws=ws)
         ys = None
@@ -303,7 +309,7 @@ class MoeTopKSigmoid(FeedForward):
             ys = ws.take((T, d), torch.float32)
             linear(act_s, self.ws_down, ys, ws=ws)
         out = ws.take((T, d), torch.float32)
-        hipops.moe_combine(y, weight, ys, out, T, k)
+        hipops.moe_combine(y, None if self.weight_input else weight, ys, out, T, k)
         return (out,)
 
 

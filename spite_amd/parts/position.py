@@ -13,6 +13,10 @@ pairs that turn often keep theirs, slow pairs are stretched; sine and cosine are
 the ``magnitude`` 0.1 ln(factor) + 1 (a mixer whose kernel knows no magnitude refuses the encoding).  The
 table is computed in float64 and stored as fp32; angle and rotation are fp32 in the kernel.
 
+``distance_slopes``: nothing is done to q and k; head h's score of (query at i, key at j) loses
+slope_h * (i - j) with slope_h = 2^(-ratio (h + 1) / H), H the number of heads: the further a key, the less it counts,
+each head at its own rate.
+
 ``none``: no position information (NoPE layers).
 """
 from __future__ import annotations
@@ -96,3 +100,15 @@ class NoPosition(PositionEncoding):
 
     def __init__(self, env):
         pass
+
+
+@register("position", "distance_slopes")
+class DistanceSlopes(PositionEncoding):
+    graph_safe = True
+
+    def __init__(self, env, ratio: float = 8.0):
+        self.env, self.ratio = env, float(ratio)
+
+    def score_slopes(self, n_heads: int):
+        vals = [2.0 ** (-self.ratio * (h + 1) / n_heads) for h in range(n_heads)]
+        return torch.tensor(vals, dtype=torch.float64).to(torch.float32).to(self.env.device)

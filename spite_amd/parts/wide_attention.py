@@ -19,7 +19,17 @@ keys and queries ``key_dim`` wide, values ``value_dim`` wide, with, each as an o
   projection;
 * ``sinks``: every head's softmax has one more term in its denominator, exp(s_h) with a learned number
   s_h per head (``sink`` [H]): it is no key, is not scaled, brings no value and counts once, so a head
-  may give less than all of its weight to the keys it sees.
+  may give less than all of its weight to the keys it sees; ``sinks="zero"``: the term is exp(0) = 1 for
+  every head and no tensor holds it;
+* ``conv_taps`` > 1: a short causal convolution over time on every channel of the q and of the k projection
+  (``q_conv`` [H*key_dim, taps], ``k_conv`` [G*key_dim, taps], the last column the token's own), right after the
+  projection; the last taps - 1 projected rows of a request are its state between steps;
+* ``head_norm``: an RMS norm of every q and k head on its own, with one weight vector for all heads
+  (``q_norm``, ``k_norm`` [key_dim]);
+* ``q_temperature`` = (coef, every): the normed queries at position p times 1 + coef ln(floor((p+1)/every) + 1);
+* ``values="keys"``: there is no value projection; the values are the keys as they leave the convolution,
+  before their norm (``value_dim`` = ``key_dim``);
+* ``score_position``: a position part that works on the scores (per-head slopes on the distance).
 
 Inside, two maps are 2H query heads over 2G key heads over G value heads: the projections' rows
 are reordered map by map when they are loaded, so that query head m*H + h reads key head
@@ -45,7 +55,8 @@ class WideAttention(Mixer):
 
     def __init__(self, env, hidden_size, n_heads, n_kv_heads, key_dim, value_dim, scale, position=None,
                  value_position=None, visibility="full", span=0, bias=False, projection_norm=False, norm_eps=1e-5,
-                 maps=1, diff=0.0, head_gate=False, sinks=False):
+                 maps=1, diff=0.0, head_gate=False, sinks=False, conv_taps=0, head_norm=False, q_temperature=None,
+                 values="projection", score_position=None):
         if n_heads % n_kv_heads:
             raise ValueError(f"wide_attention: {n_heads} heads over {n_kv_heads} kv heads")
         if visibility not in hipops.VIS:
@@ -56,6 +67,16 @@ class WideAttention(Mixer):
             raise ValueError(f"wide_attention: {maps} score maps a head")
         if maps == 2 and (value_position is not None or head_gate or sinks):
             raise ValueError("wide_attention: two score maps go with neither turned values nor a head gate nor sinks")
+        if values not in ("projection", "keys"):
+            raise ValueError(f"wide_attention: values {values!r} (known: projection, keys)")
+        if values == "keys" and (int(value_dim) != int(key_dim) or maps != 1 or value_position is not None or bias):
+            raise ValueError("wide_attention: values taken from the keys have the keys' width, one map, no rotation, no bias")
+        if head_norm and projection_norm:
+            raise ValueError("wide_attention: a norm per head or one over the whole projection, not both")
+        if (conv_taps or 0) > 1 and (maps != 1 or bias):
+            raise ValueError("wide_attention: the convolution goes with one map and no biases")
+        if sinks not in (False, True, None, "zero"):
+            raise ValueError(f"wide_attention: sinks {sinks!r} (known: True, 'zero')")
         self.env = env
         self.d, self.H, self.G = int(hidden_size), int(n_heads), int(n_kv_heads)
         self.D, self.Vd, self.maps = int(key_dim), int(value_dim), int(maps)
@@ -63,7 +84,15 @@ class WideAttention(Mixer):
         self.visibility, self.span = visibility, int(span or 0)
         self.bias, self.projection_norm, self.head_gate = bool(bias), bool(projection_norm), bool(head_gate)
         self.sinks = bool(sinks)
+        self.zero_sinks = sinks == "zero"
         self.w_sink = None
+        self.taps = int(conv_taps or 0) if int(conv_taps or 0) > 1 else 0
+        self.head_norm, self.values_from_keys = bool(head_norm), values == "keys"
+        self.q_temperature = None if not q_temperature else (float(q_temperature[0]), int(q_temperature[1]))
+        if self.q_temperature is not None and self.q_temperature[1] < 1:
+            raise ValueError(f"wide_attention: query temperature every {self.q_temperature[1]} positions")
+        self.score_position = build_part("position", score_position, env) if score_position is not None else None
+        self.slopes = self.w_conv = None
         self.position = build_part("position", position, env) if position is not None else None
         self.value_position = build_part("position", value_position, env) if value_position is not None else None
         for pe in (self.position, self.value_position):
@@ -75,7 +104,8 @@ class WideAttention(Mixer):
         self.Dk = self.D
         if env.dtype == torch.bfloat16 and self.Vd in (64, 128) and self.D < self.Vd and self.HQ // self.GK <= 16:
             self.Dk = self.Vd
-        self.n_qkv = (self.HQ + self.GK) * self.D + self.G * self.Vd
+        self.n_qk = (self.HQ + self.GK) * self.D
+        self.n_qkv = self.n_qk + (0 if self.values_from_keys else self.G * self.Vd)
         self.w_in = self.wo = self.b_in = self.w_qnorm = self.w_knorm = None
         self.inv_freq = self.inv_freq_v = None
         self.rot = 0
@@ -85,8 +115,14 @@ class WideAttention(Mixer):
     # ------------------------------------------------------------------ tensors
     def params(self):
         d, H, G, D, Vd, m = self.d, self.H, self.G, self.D, self.Vd, self.maps
-        p = {"q_proj": ParamSpec((H * m * D, d)), "k_proj": ParamSpec((G * m * D, d)), "v_proj": ParamSpec((G * Vd, d)),
-             "o_proj": ParamSpec((d, H * Vd))}
+        p = {"q_proj": ParamSpec((H * m * D, d)), "k_proj": ParamSpec((G * m * D, d)), "o_proj": ParamSpec((d, H * Vd))}
+        if not self.values_from_keys:
+            p["v_proj"] = ParamSpec((G * Vd, d))
+        if self.taps:
+            p.update({"q_conv": ParamSpec((H * D, self.taps), kind="vector", init="normal"),
+                      "k_conv": ParamSpec((G * D, self.taps), kind="vector", init="normal")})
+        if self.head_norm:
+            p.update({"q_norm": ParamSpec((D,), kind="vector", init="ones"), "k_norm": ParamSpec((D,), kind="vector", init="ones")})
         if self.bias:
             p.update({"q_bias": ParamSpec((H * m * D,), kind="vector", init="normal"),
                       "k_bias": ParamSpec((G * m * D,), kind="vector", init="normal"),
@@ -98,7 +134,7 @@ class WideAttention(Mixer):
             p.update({k: ParamSpec((D,), kind="vector", init="normal") for k in ("lambda_q1", "lambda_k1", "lambda_q2", "lambda_k2")})
         if self.head_gate:
             p["gate_proj"] = ParamSpec((H, d))
-        if self.sinks:
+        if self.sinks and not self.zero_sinks:
             p["sink"] = ParamSpec((H,), kind="vector", init="normal")
         return p
 
@@ -111,7 +147,7 @@ class WideAttention(Mixer):
 
     def load(self, t):
         H, G = self.H, self.G
-        mats = [self._by_map(t["q_proj"], H), self._by_map(t["k_proj"], G), t["v_proj"]]
+        mats = [self._by_map(t["q_proj"], H), self._by_map(t["k_proj"], G)] + ([] if self.values_from_keys else [t["v_proj"]])
         if self.head_gate:
             mats.append(t["gate_proj"])
         dts = {m.dtype for m in mats}
@@ -125,13 +161,18 @@ class WideAttention(Mixer):
         self.wo = Weight(t["o_proj"])
         if self.bias:
             self.b_in = torch.cat([self._by_map(t["q_bias"], H), self._by_map(t["k_bias"], G), t["v_bias"]]).float().contiguous()
-        if self.projection_norm:
+        if self.projection_norm or self.head_norm:
             self.w_qnorm, self.w_knorm = t["q_norm"].float().contiguous(), t["k_norm"].float().contiguous()
+        if self.taps:
+            self.w_conv = torch.cat([t["q_conv"].float(), t["k_conv"].float()], dim=0).contiguous()
+        if self.score_position is not None:
+            self.slopes = self.score_position.score_slopes(self.HQ)
         if self.maps == 2:
             dot = lambda a, b: float((t[a].double() * t[b].double()).sum())
             self.lam = math.exp(dot("lambda_q1", "lambda_k1")) - math.exp(dot("lambda_q2", "lambda_k2")) + self.diff
         if self.sinks:
-            self.w_sink = t["sink"].float().contiguous()
+            self.w_sink = torch.zeros(H, dtype=torch.float32, device=self.env.device) if self.zero_sinks \
+                else t["sink"].float().contiguous()
         if self.position is not None:
             ka = self.position.kernel_args()
             if ka["use_rope"]:
@@ -158,7 +199,11 @@ class WideAttention(Mixer):
         return notes
 
     def cache_need(self):
-        return CacheNeed(kv=KVNeed(self.GK, self.Dk, self.visibility, self.span, v_head_dim=self.Vd, n_v_heads=self.G))
+        from .base import StateNeed
+        # with a convolution: the last taps - 1 projected q and k rows of the request, fp32
+        state = StateNeed((self.taps - 1, self.n_qk), torch.float32) if self.taps else None
+        return CacheNeed(kv=KVNeed(self.GK, self.Dk, self.visibility, self.span, v_head_dim=self.Vd, n_v_heads=self.G),
+                         state=state)
 
     def _mfma(self, page_size):
         return (self.env.dtype == torch.bfloat16 and self.Dk == self.Vd and self.Vd in (64, 128) and page_size % 32 == 0
@@ -175,7 +220,7 @@ class WideAttention(Mixer):
         scratch = ctx.ws.take((hipops.attn_decode_workspace(T, HQ, D, n_splits) // 4,), torch.float32)
         hipops.attn_decode(q, cache.k_pages, cache.v_pages, o, scratch, ctx.positions, ctx.seq_of_token,
                            cache.block_table, T, HQ, GK, D, cache.page_size, self.visibility, self.span,
-                           self.scale, n_splits, value_heads=self.G, sinks=self.w_sink)
+                           self.scale, n_splits, value_heads=self.G, sinks=self.w_sink, slopes=self.slopes)
 
     def _prefill(self, q, o, ctx, cache, lead, cu_seqlens):
         HQ, GK, D = self.HQ, self.GK, self.Dk
@@ -189,18 +234,27 @@ class WideAttention(Mixer):
             scratch = ctx.ws.take((hipops.attn_prefill_workspace(counts, HQ, GK, D, n_splits) // 4,), torch.float32)
         hipops.attn_prefill(q, cache.k_pages, cache.v_pages, o, ctx.positions[lead:], cu_seqlens, counts,
                             cache.block_table[lead:], HQ, GK, D, cache.page_size, self.visibility, self.span, self.scale,
-                            n_splits=n_splits, scratch=scratch, value_heads=self.G, sinks=self.w_sink)
+                            n_splits=n_splits, scratch=scratch, value_heads=self.G, sinks=self.w_sink, slopes=self.slopes)
 
     def forward(self, x, ctx, cache):
         T, ws = x.shape[0], ctx.ws
         H, G, HQ, GK, D, Vd, Dk = self.H, self.G, self.HQ, self.GK, self.D, self.Vd, self.Dk
         proj = ws.take((T, self.n_in), x.dtype)
         linear(x, self.w_in, proj, ws=ws)
+        conv = None
+        if self.taps:
+            # (with values taken from the keys the convolved rows are all that the next kernel reads)
+            if not self.values_from_keys:
+                raise hipops.KernelError("wide_attention: the convolution goes with values taken from the keys")
+            conv = ws.take((T, self.n_qk), x.dtype)
+            hipops.causal_conv(proj[:, :self.n_qk], self.w_conv, conv, cache.state, ctx.seq_of_token, ctx.cu_seqlens,
+                               ctx.seq_slots, keep=cache.write)
         q = ws.take((T, HQ * Dk), x.dtype)
-        hipops.qkv_prepare(proj, q, cache.k_pages, cache.v_pages, ctx.positions, cache.slot_map, HQ, GK, G, D, Vd,
+        hipops.qkv_prepare(conv if self.taps else proj, q, cache.k_pages, cache.v_pages, ctx.positions, cache.slot_map, HQ, GK, G, D, Vd,
                            cache.page_size, bias=self.b_in, norm_q=self.w_qnorm, norm_k=self.w_knorm, eps=self.eps,
                            inv_freq=self.inv_freq, rot=self.rot, inv_freq_v=self.inv_freq_v, write_kv=cache.write,
-                           k_tiled=cache.tiled, v_tiled=cache.tiled, stored_dim=Dk, rot_magnitude=self.rot_magnitude)
+                           k_tiled=cache.tiled, v_tiled=cache.tiled, stored_dim=Dk, rot_magnitude=self.rot_magnitude,
+                           head_norm=self.head_norm, q_temperature=self.q_temperature, values_from_keys=self.values_from_keys)
         if cache.tiled and self._mfma(cache.page_size):
             a = ws.take((T, HQ * Vd), x.dtype)
             cu_tail, lead = ctx.derived[TAIL]
@@ -215,7 +269,7 @@ class WideAttention(Mixer):
             a = ws.take((T, HQ * Vd), torch.float32 if self.maps == 2 else x.dtype)
             hipops.attn_wide(q, cache.k_pages, cache.v_pages, a, ctx.positions, ctx.seq_of_token, cache.block_table,
                              T, HQ, GK, G, Dk, Vd, cache.page_size, self.visibility, self.span, self.scale,
-                             k_tiled=cache.tiled, v_tiled=cache.tiled, sinks=self.w_sink)
+                             k_tiled=cache.tiled, v_tiled=cache.tiled, sinks=self.w_sink, slopes=self.slopes)
         if self.maps == 2 or self.inv_freq_v is not None or self.head_gate:
             o = ws.take((T, H * Vd), x.dtype)
             gate = proj[:, self.n_qkv:self.n_qkv + H] if self.head_gate else None
