@@ -30,7 +30,7 @@ def _attention(d, a, p, eps, plain):
         names.update({"q_norm": p + "q.norm", "k_norm": p + "k.norm"})
         args.update(head_norm=True, values="keys", sinks="zero", q_temperature=a.q_temp,
                     score_position=PartSpec("distance_slopes", {"ratio": 8.0}))
-        if a.conv > 1:
+        if a.conv >= 1:
             names.update({"q_conv": p + "q.conv", "k_conv": p + "k.conv"})
             args.update(conv_taps=a.conv)
     else:

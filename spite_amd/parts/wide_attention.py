@@ -21,7 +21,7 @@ keys and queries ``key_dim`` wide, values ``value_dim`` wide, with, each as an o
   s_h per head (``sink`` [H]): it is no key, is not scaled, brings no value and counts once, so a head
   may give less than all of its weight to the keys it sees; ``sinks="zero"``: the term is exp(0) = 1 for
   every head and no tensor holds it;
-* ``conv_taps`` > 1: a short causal convolution over time on every channel of the q and of the k projection
+* ``conv_taps`` >= 1: a short causal convolution over time on every channel of the q and of the k projection
   (``q_conv`` [H*key_dim, taps], ``k_conv`` [G*key_dim, taps], the last column the token's own), right after the
   projection; the last taps - 1 projected rows of a request are its state between steps;
 * ``head_norm``: an RMS norm of every q and k head on its own, with one weight vector for all heads
@@ -73,8 +73,8 @@ class WideAttention(Mixer):
             raise ValueError("wide_attention: values taken from the keys have the keys' width, one map, no rotation, no bias")
         if head_norm and projection_norm:
             raise ValueError("wide_attention: a norm per head or one over the whole projection, not both")
-        if (conv_taps or 0) > 1 and (maps != 1 or bias):
-            raise ValueError("wide_attention: the convolution goes with one map and no biases")
+        if (conv_taps or 0) >= 1 and (maps != 1 or bias or values != "keys"):
+            raise ValueError("wide_attention: the convolution goes with one map, no biases and values taken from the keys")
         if sinks not in (False, True, None, "zero"):
             raise ValueError(f"wide_attention: sinks {sinks!r} (known: True, 'zero')")
         self.env = env
@@ -86,7 +86,7 @@ class WideAttention(Mixer):
         self.sinks = bool(sinks)
         self.zero_sinks = sinks == "zero"
         self.w_sink = None
-        self.taps = int(conv_taps or 0) if int(conv_taps or 0) > 1 else 0
+        self.taps = max(int(conv_taps or 0), 0)             # 1: a weight per channel on the token's own row, no state
         self.head_norm, self.values_from_keys = bool(head_norm), values == "keys"
         self.q_temperature = None if not q_temperature else (float(q_temperature[0]), int(q_temperature[1]))
         if self.q_temperature is not None and self.q_temperature[1] < 1:
@@ -201,7 +201,7 @@ class WideAttention(Mixer):
     def cache_need(self):
         from .base import StateNeed
         # with a convolution: the last taps - 1 projected q and k rows of the request, fp32
-        state = StateNeed((self.taps - 1, self.n_qk), torch.float32) if self.taps else None
+        state = StateNeed((self.taps - 1, self.n_qk), torch.float32) if self.taps > 1 else None
         return CacheNeed(kv=KVNeed(self.GK, self.Dk, self.visibility, self.span, v_head_dim=self.Vd, n_v_heads=self.G),
                          state=state)
 
@@ -244,8 +244,6 @@ class WideAttention(Mixer):
         conv = None
         if self.taps:
             # (with values taken from the keys the convolved rows are all that the next kernel reads)
-            if not self.values_from_keys:
-                raise hipops.KernelError("wide_attention: the convolution goes with values taken from the keys")
             conv = ws.take((T, self.n_qk), x.dtype)
             hipops.causal_conv(proj[:, :self.n_qk], self.w_conv, conv, cache.state, ctx.seq_of_token, ctx.cu_seqlens,
                                ctx.seq_slots, keep=cache.write)

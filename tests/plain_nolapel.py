@@ -91,8 +91,9 @@ def conv_attention(n, W, p, mx, eps):
     temperature that grows with the position, a distance bias, a window, a sink of score 0."""
     T = n.shape[0]
     H, G, D = mx["heads"], mx["kv_heads"], mx["dim"]
-    q = causal_conv(n @ W[p + "q"].T, W[p + "q.conv"])
-    k = causal_conv(n @ W[p + "k"].T, W[p + "k.conv"])
+    q, k = n @ W[p + "q"].T, n @ W[p + "k"].T
+    if mx.get("conv"):
+        q, k = causal_conv(q, W[p + "q.conv"]), causal_conv(k, W[p + "k.conv"])
     v = k.view(T, G, D)
     q = unit_rms(q.view(T, H, D), eps) * W[p + "q.norm"]
     k = unit_rms(k.view(T, G, D), eps) * W[p + "k.norm"]
