@@ -169,7 +169,10 @@ class KernelTimes:
              "attn_generic", "gemm_skinny", "gemm_mfma", "gemm_tiled", "attn_decode", "attn_prefill",
              "sample_rows", "argmax_rows", "filter_rows", "latent_prepare", "attn_latent_generic", "attn_latent_mfma",
              "router_topk", "moe_combine", "gated_rows", "add_into",
-             "qkv_prepare", "attn_wide", "attn_finish", "token_shift", "act_rows")
+             "qkv_prepare", "attn_wide", "attn_finish", "token_shift", "act_rows",
+             "linear_attn_scan", "channel_decay", "gated_group_norm", "scale_rows",
+             "add_tanh_norm", "hash_rows", "embed_sum", "causal_conv", "shift_mix", "step_decay", "softcap_rows",
+             "axpby_rows", "concat_rows", "bias_rows")
 
     def __init__(self):
         import torch
@@ -228,6 +231,13 @@ class KernelTimes:
 # heads x 128 x 128 numbers a request; softmax attention with sinks, heads of 128, a kv head for every four, the first
 # 64 elements turning with YaRN-scaled frequencies, chunks of 4,096), every layer with the experts of the size, their
 # shared expert and per-layer token rows of 256.
+# ``--design nolapel``: the Nolapel design beside Tebalorn (the closest existing design: recurrent states, attention
+# with sinks, several experts a token).  Nolapel: layers in the order mamba2, attention, parallel, mamba2 (a state-space mixer
+# with heads of 128 values over 128 state channels, a group for every eight heads, a convolution of four taps; attention
+# whose values are its keys, heads of 128, a kv head for every four, a convolution of four taps, a window of 4,096;
+# attention with learned sinks and 64 turning elements beside time mixing with heads of 128), tanh norms before and
+# after every sublayer, the first two layers behind a reentry product (a loop walked once), the hashed pair
+# embedding, the experts of the size weighted at their input, their shared expert.
 DESIGN_SIZES = {
     "2k": dict(width=2048, heads=16, experts=16, top=4, expert_ff=1024, shared_ff=2048, dense_ff=8192),
     "5k": dict(width=5120, heads=40, experts=16, top=2, expert_ff=4096, shared_ff=8192, dense_ff=16384),
@@ -274,7 +284,28 @@ def tebalorn_configs(sz, layers, window, vocab):
     return {"tebalorn": tebalorn, "llama4": llama}
 
 
+def nolapel_configs(sz, layers, window, vocab):
+    H = sz["heads"]
+    groups = max(1, H // 8)
+    ssm = ("mamba2", {"heads": H, "vdim": 128, "state": 128, "groups": groups, "conv": 4, "norm_groups": groups})
+    attn = ("attention", {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
+                          "mask": {"size": window}, "q_temp": {"coef": 0.3, "every": 1024}})
+    par = ("parallel", {"left": {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                 "rot": {"base": 1000000.0, "dims": 64}},
+                        "right": {"heads": H, "dim": 128}, "left_scale": 1.2, "right_scale": 0.9})
+    mixers = [ssm, attn, par, ssm]
+    mlp = {"kind": "moe", "router": {"experts": sz["experts"], "top": sz["top"]}, "expert": {"ff": sz["expert_ff"]},
+           "shared": {"ff": sz["shared_ff"]}}
+    nolapel = {"architecture": "Nolapel", "vocab": vocab, "width": sz["width"], "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+               "embedding": {"bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 17}}, "torch_dtype": "bfloat16",
+               "loop": {"start": 0, "stop": min(2, layers), "times": 1},
+               "layers": [{"type": mixers[i % 4][0], "mixer": mixers[i % 4][1], "mlp": mlp} for i in range(layers)]}
+    return {"nolapel": nolapel, "tebalorn": tebalorn_configs(sz, layers, window, vocab)["tebalorn"]}
+
+
 def design_configs(sz, layers, window, vocab, design="ravenex"):
+    if design == "nolapel":
+        return nolapel_configs(sz, layers, window, vocab)
     if design == "pefedra":
         return pefedra_configs(sz, layers, window, vocab)
     if design == "tebalorn":
@@ -307,7 +338,8 @@ def design_comparison(args):
     page, V, layers, window = 64, 32768, args.layers or 4, 4096
     batch, context, T = args.batch, args.context, args.prefill_tokens
     rng = np.random.RandomState(0)
-    out = {"metric": f"prefill and decode tok/s of the {args.design.capitalize()} design beside Llama 4 at equal sizes (random weights)",
+    beside = "Tebalorn" if args.design == "nolapel" else "Llama 4"
+    out = {"metric": f"prefill and decode tok/s of the {args.design.capitalize()} design beside {beside} at equal sizes (random weights)",
            "value": None, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": args.dtype,
            "higher_is_better": True, "data": "synthetic: random weights, uniform-random token ids, context pages filled with random values",
            "config": {"layers": layers, "window": window, "global_batch": batch, "seq_len": context, "prefill_tokens": T, "vocab": V},
@@ -635,8 +667,9 @@ def main() -> int:
     ap.add_argument("--workload", default="decode", choices=["decode", "longctx", "serve", "designs"],
                     help="designs: another design (--design) beside Llama 4 at equal sizes (see DESIGN_SIZES)")
     ap.add_argument("--design-sizes", default="2k,5k", help="designs: which of DESIGN_SIZES, comma separated")
-    ap.add_argument("--design", default="ravenex", choices=["ravenex", "pefedra", "tebalorn"],
-                    help="designs: which design runs beside Llama 4 (pefedra: against Llama 4 with dense layers only)")
+    ap.add_argument("--design", default="ravenex", choices=["ravenex", "pefedra", "tebalorn", "nolapel"],
+                    help="designs: which design runs beside Llama 4 (pefedra: against Llama 4 with dense layers only; "
+                         "nolapel: beside Tebalorn, the closest existing design)")
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (memory or time)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)

@@ -132,7 +132,10 @@ class Model:
                 state["pending"] = ()
                 ctx.ws = arenas[0]
                 estate = cache.states.get(self.embedding_cache) if self.embedding_cache is not None else None
-                self.embedding.forward(ctx.token_ids, state["h"], ctx, state=estate)
+                if estate is not None:
+                    self.embedding.forward(ctx.token_ids, state["h"], ctx, state=estate)
+                else:
+                    self.embedding.forward(ctx.token_ids, state["h"], ctx)
                 if self.spec.keep_embedding:
                     # a copy for the blocks that read the embedding's result later in the step (the norms change h in place)
                     state["h0"] = step_ws.take((ctx.T, d), torch.float32)

@@ -861,7 +861,7 @@ def test_one_far_key_stands_out_and_the_sink_counts(tmp_path, dtype, wide):
 @pytest.mark.parametrize("dtype,wide", [("float32", False), ("bfloat16", True)])
 def test_a_far_token_stays_in_the_state(tmp_path, kind, dtype, wide):
     """Decays next to 1: what the first tokens wrote into the state is still read hundreds of tokens later, through a
-    long prompt in one step and more than a hundred tokens decoded one by one.  Changing tokens 1 to 8 moves the last logits
+    long prompt in one step and more than a hundred tokens decoded one by one.  Changing tokens 1 to 80 moves the last logits
     of the plain implementation, and the engine follows it at every position."""
     if kind == "time_mix":
         mixer = _parallel(2, 1, 64, 64, 0.1, None, 2, 64, ls=0.05, rs=1.0) if wide else _parallel(1, 1, 4, 4, 0.1, None, 3, 6, ls=0.05, rs=1.0)
@@ -879,7 +879,7 @@ def test_a_far_token_stays_in_the_state(tmp_path, kind, dtype, wide):
     weights = H.read_weights(str(tmp_path))
     toks = H.random_tokens(64, 420, 6)
     other = list(toks)
-    for j in range(1, 9):
+    for j in range(1, 81):
         other[j] = (toks[j] + 5) % 64
     ref = plain.forward(toks, weights, cfg)
     scale = float(ref.abs().max())
