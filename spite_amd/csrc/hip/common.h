@@ -127,6 +127,27 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return t;
 }
 
+// ------------------------------------------------------------------ a wave's fp32 dot product
+// sum_c w[c] * xs[c] over a row xs in LDS, by one wave: lane l takes the 16-byte groups l, l+64,
+// ... and the lanes' sums meet in a butterfly.  Every kernel that forms router logits calls
+// this, so a logit has the same bits wherever it is computed; its order of summation depends
+// on the width alone.
+__device__ __forceinline__ float wave_dot_row(const float* __restrict__ w, const float* xs, int d, bool vec, int lane) {
+    float acc = 0.f;
+    if (vec) {
+        const int nv = d >> 2;
+#pragma unroll 10
+        for (int c = lane; c < nv; c += 64) {          // independent 16-byte loads, ten in flight
+            const f32x4 ww = ((const f32x4*)w)[c];
+            const f32x4 xx = ((const f32x4*)xs)[c];
+            acc += ww[0] * xx[0] + ww[1] * xx[1] + ww[2] * xx[2] + ww[3] * xx[3];
+        }
+    } else {
+        for (int c = lane; c < d; c += 64) acc += w[c] * xs[c];
+    }
+    return wave_sum(acc);
+}
+
 // The gate's activation in a gated product act(gate) * up: SP_ACT_SILU g * sigmoid(g),
 // SP_ACT_GELU_TANH 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))), or SP_ACT_RELU max(g, 0).
 // `fast`: the short exponential (the bfloat16 products); the 32-bit path takes the accurate routines.

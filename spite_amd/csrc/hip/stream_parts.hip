@@ -84,6 +84,74 @@ void add_tanh_norm_any_kernel(float* __restrict__ h, const float* __restrict__ d
     }
 }
 
+// The same with small fp32 products of the normed row formed on the way (router logits): a workgroup a row, the
+// normed row kept in LDS, proj_out[i][e] = proj[e] . normed row, a wave a product.  Rows of a multiple of four
+// elements that fit the LDS.
+template <typename TO>
+__global__ __launch_bounds__(256)
+void add_tanh_norm_proj_kernel(float* __restrict__ h, const float* __restrict__ d1, const float* __restrict__ d2,
+                               const float* __restrict__ yn, const float* __restrict__ wn, const float* __restrict__ bn,
+                               const float* __restrict__ alpha_n, float mult,
+                               const float* __restrict__ w, const float* __restrict__ b, const float* __restrict__ alpha,
+                               TO* __restrict__ out, float* __restrict__ out32, int d, int write_h,
+                               const float* __restrict__ proj, float* __restrict__ proj_out, int P) {
+    extern __shared__ __attribute__((aligned(16))) float xs[];
+    const size_t r = blockIdx.x;
+    const float a = alpha[0], an = alpha_n ? alpha_n[0] : 0.f;
+    for (int c = threadIdx.x * 4; c < d; c += 1024) {
+        f32x4 v = *(const f32x4*)(h + r * d + c);
+        if (d1) v += *(const f32x4*)(d1 + r * d + c);
+        if (d2) v += *(const f32x4*)(d2 + r * d + c);
+        if (yn) {
+            const f32x4 y = *(const f32x4*)(yn + r * d + c), ww = *(const f32x4*)(wn + c), bb = *(const f32x4*)(bn + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += mult * fmaf(tanhf(an * y[e]), ww[e], bb[e]);
+        }
+        if (write_h) *(f32x4*)(h + r * d + c) = v;
+        const f32x4 ww = *(const f32x4*)(w + c), bb = *(const f32x4*)(b + c);
+        f32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = fmaf(tanhf(a * v[e]), ww[e], bb[e]);
+        *(f32x4*)(xs + c) = o;
+        if (out) {
+            if constexpr (sizeof(TO) == 2) {
+                const bf16x4 o4 = {(bf16)o[0], (bf16)o[1], (bf16)o[2], (bf16)o[3]};
+                *(bf16x4*)((bf16*)out + r * d + c) = o4;
+            } else {
+                *(f32x4*)((float*)out + r * d + c) = o;
+            }
+        }
+        if (out32) *(f32x4*)(out32 + r * d + c) = o;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    for (int e = threadIdx.x >> 6; e < P; e += 4) {
+        const float s = wave_dot_row(proj + (size_t)e * d, xs, d, true, lane);
+        if (lane == 0) proj_out[r * P + e] = s;
+    }
+}
+
+extern "C" int spite_add_tanh_norm_proj(float* h, const float* d1, const float* d2, const float* yn, const float* wn,
+                                        const float* bn, const float* alpha_n, float mult, const float* w, const float* b,
+                                        const float* alpha, void* out, int out_dtype, float* out32, int n_rows, int d,
+                                        int write_h, const float* proj, float* proj_out, int P, hipStream_t st) {
+    SP_REQUIRE(n_rows >= 0 && d > 0 && d % 4 == 0 && (size_t)d * 4 <= 48 * 1024 && P > 0, "add_tanh_norm: rows of %d with %d products", d, P);
+    SP_REQUIRE(!yn || (wn && bn && alpha_n), "add_tanh_norm: a normed increment needs its weight, bias and alpha");
+    SP_REQUIRE(w && b && alpha && proj && proj_out, "add_tanh_norm: the products need the norm and their matrix");
+    if (n_rows == 0) return 0;
+    auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    SP_REQUIRE(al(h) && al(d1) && al(d2) && al(yn) && al(wn) && al(bn) && al(w) && al(b) && al(out32) && al(proj)
+               && (out_dtype == SP_F32 ? al(out) : ((uintptr_t)out & 7) == 0), "add_tanh_norm: rows must start on 16 bytes");
+    const size_t sh = (size_t)d * sizeof(float);
+#define SP_TNP(TO) add_tanh_norm_proj_kernel<TO><<<n_rows, 256, sh, st>>>(h, d1, d2, yn, wn, bn, alpha_n, mult, w, b, alpha, (TO*)out, out32, d, write_h, proj, proj_out, P)
+    if (out_dtype == SP_F32) SP_TNP(float);
+    else if (out_dtype == SP_BF16) SP_TNP(bf16);
+    else return sp_fail("add_tanh_norm: unknown dtype %d", out_dtype);
+#undef SP_TNP
+    SP_LAUNCH_CHECK("add_tanh_norm");
+    return 0;
+}
+
 extern "C" int spite_add_tanh_norm(float* h, const float* d1, const float* d2, const float* yn, const float* wn,
                                    const float* bn, const float* alpha_n, float mult, const float* w, const float* b,
                                    const float* alpha, void* out, int out_dtype, float* out32, const int* rows,
@@ -221,6 +289,62 @@ void causal_conv_kernel(const TI* __restrict__ x, int ldx, const float* __restri
     }
 }
 
+// bfloat16 rows whose sizes let a thread take eight channels at a time (16-byte loads and stores).  The thread of an
+// entry's token further than taps - 2 into the entry reads rows of the step only; the others leave their eight
+// channels to the one-channel kernel's rule (see above), applied here channel by channel.
+#define CONV_VEC_TAPS 8
+__global__ __launch_bounds__(256)
+void causal_conv_vec_kernel(const bf16* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ bias,
+                            float* __restrict__ state, const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
+                            const int* __restrict__ seq_slots, bf16* __restrict__ y, int ldy, int C, int taps, int act, int keep) {
+    const int t = blockIdx.x;
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+    if (c >= C) return;
+    const int e = seq_of_token[t];
+    const int first = cu_seqlens[e], end = cu_seqlens[e + 1];
+    const int local = t - first, back = taps - 1;
+    auto finish = [&](float v) { return act == 1 ? v / (1.0f + expf(-v)) : v; };
+    if (local >= back) {
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = bias ? bias[c + i] : 0.f;
+#pragma unroll
+        for (int j = 0; j < CONV_VEC_TAPS; ++j) {
+            if (j < taps) {
+                const bf16x8 xv = *(const bf16x8*)(x + (size_t)(t - back + j) * ldx + c);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[i] = fmaf(w[(size_t)(c + i) * taps + j], (float)xv[i], acc[i]);
+            }
+        }
+        bf16x8 o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (bf16)finish(acc[i]);
+        *(bf16x8*)(y + (size_t)t * ldy + c) = o;
+        return;
+    }
+    if (local != 0) return;
+    const int count = end - first;
+    const int n_here = count < back ? count : back;
+    for (int i = 0; i < 8; ++i) {
+        const int ci = c + i;
+        float* sr = state + (size_t)seq_slots[e] * back * C + ci;
+        float old[CONV_VEC_TAPS];
+        for (int k = 0; k < back; ++k) old[k] = sr[(size_t)k * C];
+        auto z = [&](int idx) { return idx < back ? old[idx] : (float)x[(size_t)(first + idx - back) * ldx + ci]; };
+        const float b0 = bias ? bias[ci] : 0.f;
+        for (int m = 0; m < n_here; ++m) {
+            float acc = b0;
+            for (int j = 0; j < taps; ++j) acc = fmaf(w[(size_t)ci * taps + j], z(m + j), acc);
+            y[(size_t)(first + m) * ldy + ci] = (bf16)finish(acc);
+        }
+        if (keep) {
+            float keep_v[CONV_VEC_TAPS];
+            for (int k = 0; k < back; ++k) keep_v[k] = z(count + k);
+            for (int k = 0; k < back; ++k) sr[(size_t)k * C] = keep_v[k];
+        }
+    }
+}
+
 extern "C" int spite_causal_conv(const void* x, int ldx, int x_dtype, const float* w, const float* bias, float* state,
                                  const int* seq_of_token, const int* cu_seqlens, const int* seq_slots, void* y, int ldy,
                                  int y_dtype, int T, int C, int taps, int act, int keep, hipStream_t st) {
@@ -228,6 +352,14 @@ extern "C" int spite_causal_conv(const void* x, int ldx, int x_dtype, const floa
     SP_REQUIRE(ldx >= C && ldy >= C && (act == 0 || act == 1), "causal_conv: rows shorter than the channels, or activation %d", act);
     SP_REQUIRE(taps == 1 || state, "causal_conv: the request's last inputs need a state");
     if (T == 0) return 0;
+    if (x_dtype == SP_BF16 && y_dtype == SP_BF16 && C % 8 == 0 && ldx % 8 == 0 && ldy % 8 == 0 && taps <= CONV_VEC_TAPS
+        && ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 15) == 0) {
+        const dim3 vgrid(T, (C / 8 + 255) / 256);
+        causal_conv_vec_kernel<<<vgrid, 256, 0, st>>>((const bf16*)x, ldx, w, bias, state, seq_of_token, cu_seqlens, seq_slots,
+                                                      (bf16*)y, ldy, C, taps, act, keep);
+        SP_LAUNCH_CHECK("causal_conv");
+        return 0;
+    }
     const dim3 grid(T, (C + 255) / 256);
     SP_REQUIRE(grid.y <= 65535, "causal_conv: too many channels");
 #define SP_CC(TI, TO) causal_conv_kernel<TI, TO><<<grid, 256, 0, st>>>((const TI*)x, ldx, w, bias, state, seq_of_token, cu_seqlens, \
@@ -267,10 +399,58 @@ void shift_mix_kernel(const T* __restrict__ x, const float* __restrict__ mu, flo
     }
 }
 
+// bfloat16 rows of a multiple of eight elements: eight elements a thread, 16-byte loads and stores.
+__global__ __launch_bounds__(256)
+void shift_mix_vec_kernel(const bf16* __restrict__ x, const float* __restrict__ mu, float* __restrict__ state, bf16* __restrict__ y,
+                          const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
+                          const int* __restrict__ seq_slots, int Tn, int d, int n, int keep) {
+    const int t = blockIdx.x;
+    const int e = seq_of_token[t];
+    const int first = cu_seqlens[e], last = cu_seqlens[e + 1] - 1;
+    for (int c = (blockIdx.y * 256 + threadIdx.x) * 8; c < d; c += gridDim.y * 2048) {
+        const bf16x8 av = *(const bf16x8*)(x + (size_t)t * d + c);
+        float a[8], before[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] = (float)av[i];
+        if (t == first) {
+            float* sr = state + (size_t)seq_slots[e] * d + c;
+            const f32x4 s0 = *(const f32x4*)sr, s1 = *(const f32x4*)(sr + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { before[i] = s0[i]; before[4 + i] = s1[i]; }
+            if (keep) {
+                const bf16x8 lv = *(const bf16x8*)(x + (size_t)last * d + c);
+                *(f32x4*)sr = f32x4{(float)lv[0], (float)lv[1], (float)lv[2], (float)lv[3]};
+                *(f32x4*)(sr + 4) = f32x4{(float)lv[4], (float)lv[5], (float)lv[6], (float)lv[7]};
+            }
+        } else {
+            const bf16x8 bv = *(const bf16x8*)(x + (size_t)(t - 1) * d + c);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) before[i] = (float)bv[i];
+        }
+        for (int s = 0; s < n; ++s) {
+            const f32x4 m0 = *(const f32x4*)(mu + (size_t)s * d + c), m1 = *(const f32x4*)(mu + (size_t)s * d + c + 4);
+            bf16x8 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                o[i] = (bf16)fmaf(before[i] - a[i], m0[i], a[i]);
+                o[4 + i] = (bf16)fmaf(before[4 + i] - a[4 + i], m1[i], a[4 + i]);
+            }
+            *(bf16x8*)(y + ((size_t)s * Tn + t) * d + c) = o;
+        }
+    }
+}
+
 extern "C" int spite_shift_mix(const void* x, int dtype, const float* mu, float* state, void* y, const int* seq_of_token,
                                const int* cu_seqlens, const int* seq_slots, int T, int d, int n, int keep, hipStream_t st) {
     SP_REQUIRE(T >= 0 && d > 0 && n > 0, "shift_mix: bad sizes T=%d d=%d n=%d", T, d, n);
     if (T == 0) return 0;
+    auto al = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    if (dtype == SP_BF16 && d % 8 == 0 && al(x) && al(y) && al(mu) && al(state)) {
+        const dim3 vgrid(T, (d / 8 + 255) / 256 < 64 ? (d / 8 + 255) / 256 : 64);
+        shift_mix_vec_kernel<<<vgrid, 256, 0, st>>>((const bf16*)x, mu, state, (bf16*)y, seq_of_token, cu_seqlens, seq_slots, T, d, n, keep);
+        SP_LAUNCH_CHECK("shift_mix");
+        return 0;
+    }
     const dim3 grid(T, (d + 255) / 256 < 64 ? (d + 255) / 256 : 64);
     if (dtype == SP_F32) shift_mix_kernel<float><<<grid, 256, 0, st>>>((const float*)x, mu, state, (float*)y, seq_of_token, cu_seqlens, seq_slots, T, d, n, keep);
     else if (dtype == SP_BF16) shift_mix_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, mu, state, (bf16*)y, seq_of_token, cu_seqlens, seq_slots, T, d, n, keep);
@@ -299,10 +479,39 @@ void step_decay_kernel(const T* __restrict__ raw, int ld, const float* __restric
     }
 }
 
+// state channels in multiples of four: a thread writes four of a head's channels in one store
+template <typename T>
+__global__ __launch_bounds__(256)
+void step_decay_vec_kernel(const T* __restrict__ raw, int ld, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                           float* __restrict__ dt, float* __restrict__ decay, int Tn, int H, int N) {
+    const int n4 = N >> 2;
+    const size_t n = (size_t)Tn * H * n4;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        const size_t th = i / n4;
+        const int ch = (int)(i - th * n4);
+        const size_t t = th / H;
+        const int h = (int)(th - t * H);
+        const float z = to_f32<T>(raw[t * ld + h]) + dt_bias[h];
+        const float step = z > 20.f ? z + log1pf(expf(-z)) : log1pf(expf(z));
+        if (ch == 0) dt[th] = step;
+        const float a = expf(-expf(a_log[h]) * step);
+        *(f32x4*)(decay + th * N + ch * 4) = f32x4{a, a, a, a};
+    }
+}
+
 extern "C" int spite_step_decay(const void* raw, int ld, int dtype, const float* dt_bias, const float* a_log, float* dt,
                                 float* decay, int T, int H, int N, hipStream_t st) {
     SP_REQUIRE(T >= 0 && H > 0 && N > 0 && ld >= H, "step_decay: bad sizes T=%d H=%d N=%d ld=%d", T, H, N, ld);
     if (T == 0) return 0;
+    if (N % 4 == 0 && ((uintptr_t)decay & 15) == 0) {
+        const size_t nv = (size_t)T * H * (N / 4);
+        const unsigned vgrid = (unsigned)((nv + 255) / 256 < 65535u * 16 ? (nv + 255) / 256 : 65535u * 16);
+        if (dtype == SP_F32) step_decay_vec_kernel<float><<<vgrid, 256, 0, st>>>((const float*)raw, ld, dt_bias, a_log, dt, decay, T, H, N);
+        else if (dtype == SP_BF16) step_decay_vec_kernel<bf16><<<vgrid, 256, 0, st>>>((const bf16*)raw, ld, dt_bias, a_log, dt, decay, T, H, N);
+        else return sp_fail("step_decay: unknown dtype %d", dtype);
+        SP_LAUNCH_CHECK("step_decay");
+        return 0;
+    }
     const size_t n = (size_t)T * H * N;
     const unsigned grid = (unsigned)((n + 255) / 256 < 65535u * 16 ? (n + 255) / 256 : 65535u * 16);
     if (dtype == SP_F32) step_decay_kernel<float><<<grid, 256, 0, st>>>((const float*)raw, ld, dt_bias, a_log, dt, decay, T, H, N);

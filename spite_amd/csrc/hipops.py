@@ -76,6 +76,7 @@ def lib():
             "spite_linear_attn_scan": [P, P, P, I, I, I, I, P, P, F, P, I, P, P, I, P, I, I, I, I, I, I, P, P, P],
             "spite_gated_group_norm": [P, P, I, P, I, P, I, I, I, I, F, I, I, P, I, P, I, P],
             "spite_add_tanh_norm": [P, P, P, P, P, P, P, F, P, P, P, P, I, P, P, I, I, I, P],
+            "spite_add_tanh_norm_proj": [P, P, P, P, P, P, P, F, P, P, P, P, I, P, I, I, I, P, P, I, P],
             "spite_hash_rows": [P, P, P, P, P, P, P, I, ctypes.c_longlong, ctypes.c_longlong, ctypes.c_longlong, I, P],
             "spite_embed_sum": [P, P, P, P, I, P, I, I, I, I, F, P],
             "spite_causal_conv": [P, I, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
@@ -1020,10 +1021,17 @@ def gated_group_norm(o, weight, y, group, eps, gate=None, act=None, gate_first=F
 
 
 # -------------------------------------------------------------------------------------------- parts around the stream
-def add_tanh_norm(h, w, b, alpha, out=None, out32=None, d1=None, d2=None, rows=None, n_rows=None, write_h=True, normed=None):
+def add_tanh_norm_can_project(d: int) -> bool:
+    """Whether ``add_tanh_norm`` forms projections of rows of this width (the row stays in LDS, four elements a thread)."""
+    return d % 4 == 0 and d * 4 <= 48 * 1024
+
+
+def add_tanh_norm(h, w, b, alpha, out=None, out32=None, d1=None, d2=None, rows=None, n_rows=None, write_h=True, normed=None,
+                  proj=None, proj_out=None):
     """h (fp32 [T,d]) += d1 + d2 + mult * (tanh(an * yn) * wn + bn) with ``normed`` = (yn, wn, bn, an, mult); then
     out[i] (and out32[i]) = tanh(alpha * h[r]) * w + b, r = rows[i] or i.  ``w`` None: out is the stream itself in
-    out's dtype.  alpha and an are fp32 tensors of one element."""
+    out's dtype.  alpha and an are fp32 tensors of one element.  ``proj`` (fp32 [P, d]) with ``proj_out`` (fp32 [T, P]):
+    proj_out[i] = proj . (the normed fp32 row i), formed in the same pass (no gathered rows then)."""
     T, d = h.shape
     n = int(n_rows if n_rows is not None else (rows.numel() if rows is not None else T))
     for name, t in (("d1", d1), ("d2", d2)):
@@ -1043,6 +1051,16 @@ def add_tanh_norm(h, w, b, alpha, out=None, out32=None, d1=None, d2=None, rows=N
         if t is not None and t.numel() < n * d:
             raise KernelError(f"add_tanh_norm: {name} too small")
     f = torch.float32
+    if proj is not None:
+        if rows is not None or w is None or proj.dim() != 2 or proj.shape[1] != d or proj_out is None or proj_out.numel() < n * proj.shape[0] \
+                or not add_tanh_norm_can_project(d):
+            raise KernelError(f"add_tanh_norm: products {None if proj is None else tuple(proj.shape)} of rows of {d}")
+        _check(lib().spite_add_tanh_norm_proj(
+            _ptr(h, "h", f), _ptr(d1, "d1", f, True), _ptr(d2, "d2", f, True), _ptr(yn, "yn", f, True), _ptr(wn, "wn", f, True),
+            _ptr(bn, "bn", f, True), _ptr(an, "an", f, True), float(mult), _ptr(w, "w", f), _ptr(b, "b", f), _ptr(alpha, "alpha", f),
+            _ptr(out, "out", None, True), dtype_code(out.dtype) if out is not None else F32, _ptr(out32, "out32", f, True), n, d,
+            int(bool(write_h)), _ptr(proj, "proj", f), _ptr(proj_out, "proj_out", f), proj.shape[0], _stream()), "add_tanh_norm")
+        return
     _check(lib().spite_add_tanh_norm(
         _ptr(h, "h", f), _ptr(d1, "d1", f, True), _ptr(d2, "d2", f, True), _ptr(yn, "yn", f, True), _ptr(wn, "wn", f, True),
         _ptr(bn, "bn", f, True), _ptr(an, "an", f, True), float(mult), _ptr(w, "w", f, True), _ptr(b, "b", f, True),

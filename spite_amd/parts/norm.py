@@ -83,9 +83,17 @@ class TanhNorm(Norm):
         from .base import TanhIncrement
         return isinstance(increment, TanhIncrement)
 
-    def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True, normed=None, plain=False):
+    def can_project(self, proj) -> bool:
+        # the kernel keeps the normed row in LDS for the products
+        return proj.dtype == torch.float32 and proj.dim() == 2 and proj.shape[1] == self.width \
+            and hipops.add_tanh_norm_can_project(self.width)
+
+    def forward(self, h, out, *, d1=None, d2=None, out32=None, rows=None, write_h=True, normed=None, plain=False,
+                proj=None, proj_out=None):
         """``normed``: a ``TanhIncrement``'s arguments, added like d1 and d2 after its own norm.  ``plain``: out is the
-        stream itself (everything added) in out's dtype, not normed."""
+        stream itself (everything added) in out's dtype, not normed.  ``proj`` / ``proj_out``: small fp32 products of
+        the normed rows formed in the same pass (router logits)."""
         w, b, a = (None, None, None) if plain else (self.weight, self.bias, self.alpha)
         hipops.add_tanh_norm(h, w, b, a, out=out, out32=out32, d1=d1, d2=d2, rows=rows,
-                             n_rows=(rows.numel() if rows is not None else h.shape[0]), write_h=write_h, normed=normed)
+                             n_rows=(rows.numel() if rows is not None else h.shape[0]), write_h=write_h, normed=normed,
+                             proj=proj, proj_out=proj_out)

@@ -362,6 +362,15 @@ def test_tanh_norm_kernel(dtype, d):
     assert torch.equal(hd, before) and float((o2.cpu().double() - want[[7, 2]]).abs().max()) < (1e-5 if dtype == "float32" else 3e-2)
     hipops.add_tanh_norm(hd, None, None, None, out=out)
     assert float((out.cpu().double() - v).abs().max()) < (1e-5 if dtype == "float32" else 3e-2)
+    if d % 4 == 0:
+        # small fp32 products of the normed rows in the same pass (router logits)
+        proj = torch.randn(5, d, generator=g)
+        h2, po = h.cuda(), torch.empty(T, 5, device="cuda:0")
+        hipops.add_tanh_norm(h2, w.cuda(), b.cuda(), al.cuda(), out=out, d1=d1.cuda(), d2=d2.cuda(),
+                             normed=(yn.cuda(), wn.cuda(), bn.cuda(), an.cuda(), 0.5), proj=proj.cuda(), proj_out=po)
+        assert float((h2.cpu().double() - v).abs().max()) < 1e-5
+        assert float((out.cpu().double() - want).abs().max()) < (1e-5 if dtype == "float32" else 3e-2)
+        assert float((po.cpu().double() - want @ proj.double().T).abs().max()) < 1e-4
 
 
 @pytest.mark.gpu
