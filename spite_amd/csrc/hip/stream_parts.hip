@@ -4,7 +4,8 @@
 //                    with one increment that passes such a norm of its own on its way into the stream
 //   hash_rows / embed_sum:  a second embedding whose row is a hash of (previous token, token); the previous token
 //                    of a request is kept in a state row
-//   causal_conv:     a short convolution over time on every channel, with the request's last inputs as state
+//   causal_conv:     a short convolution over time on every channel, with the request's last inputs as state (two
+//                    kernels: the results, then the state)
 //   shift_mix:       several blends of a row with the request's previous row, one per reader
 //   step_decay:      softplus of a step size, and the decay exp(-exp(A) dt) that it gives, spread over channels
 //   softcap_rows, axpby_rows, concat_rows, bias_rows: small fp32 row operations
@@ -236,139 +237,130 @@ extern "C" int spite_embed_sum(const int* ids, const void* table, const int* row
 }
 
 // ------------------------------------------------------------------ short convolution over time
-// y[t][c] = bias[c] + sum_j w[c][j] * u[t - taps + 1 + j][c], u before the request's first token being zero, then an
-// activation (0 none, 1 silu).  The inputs before an entry's first token are the request's state, fp32
-// [slots][taps - 1][C], oldest first, which then takes the last taps - 1 inputs of the request.  A token further than
-// taps - 2 into its entry reads rows of the step only.  The first taps - 1 tokens of an entry (the only ones that
-// need the state) are computed by the thread of the entry's first token, which also writes the new state: every
-// element of a state row is touched by one thread, so entries of any length are safe.  Sums run over j upwards from
-// the bias, the same for every token wherever a request is cut.
+// y[t][c] = bias[c] + sum_j w[j][c] * u[t - taps + 1 + j][c], u before the request's first token being zero, then an
+// activation (0 none, 1 silu).  The weights lie tap by tap, [taps][C] (the last tap is the token's own): a wave's loads
+// of one tap are consecutive.  The inputs before an entry's first token are the request's state, fp32
+// [slots][taps - 1][C], oldest first.  Every thread forms its own results, reading rows of the step where the entry
+// has them and the state where it does not; nothing writes the state here.  A second kernel (causal_conv_keep), launched
+// behind this one, then leaves the request's last taps - 1 inputs in the state: one thread reads and writes a channel's
+// state, so entries of any length are safe.  Sums run over j upwards from the bias, the same for every token wherever
+// a request is cut.
 #define CONV_MAX_TAPS 16
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256)
 void causal_conv_kernel(const TI* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ bias,
-                        float* __restrict__ state, const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
-                        const int* __restrict__ seq_slots, TO* __restrict__ y, int ldy, int C, int taps, int act, int keep) {
+                        const float* __restrict__ state, const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
+                        const int* __restrict__ seq_slots, TO* __restrict__ y, int ldy, int C, int taps, int act) {
     const int t = blockIdx.x;
     const int c = blockIdx.y * 256 + threadIdx.x;
     if (c >= C) return;
     const int e = seq_of_token[t];
-    const int first = cu_seqlens[e], end = cu_seqlens[e + 1];
+    const int first = cu_seqlens[e];
     const int local = t - first, back = taps - 1;
-    float wc[CONV_MAX_TAPS];
-#pragma unroll
-    for (int j = 0; j < CONV_MAX_TAPS; ++j) wc[j] = j < taps ? w[(size_t)c * taps + j] : 0.f;
-    const float b0 = bias ? bias[c] : 0.f;
-    auto finish = [&](float v) { return act == 1 ? v / (1.0f + expf(-v)) : v; };
-    if (local >= back) {
-        float acc = b0;
-#pragma unroll
-        for (int j = 0; j < CONV_MAX_TAPS; ++j)
-            if (j < taps) acc = fmaf(wc[j], to_f32<TI>(x[(size_t)(t - back + j) * ldx + c]), acc);
-        y[(size_t)t * ldy + c] = from_f32<TO>(finish(acc));
-        return;
+    const float* sr = state + (size_t)seq_slots[e] * back * C + c;
+    float acc = bias ? bias[c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int r = local - back + j;                    // the input's row, counted from the entry's first
+        const float u = r >= 0 ? to_f32<TI>(x[(size_t)(first + r) * ldx + c]) : sr[(size_t)(r + back) * C];
+        acc = fmaf(w[(size_t)j * C + c], u, acc);
     }
-    if (local != 0) return;
-    // z = the state's taps - 1 inputs, then the entry's
-    float* sr = state + (size_t)seq_slots[e] * back * C + c;
-    float old[CONV_MAX_TAPS];
-#pragma unroll
-    for (int i = 0; i < CONV_MAX_TAPS; ++i) old[i] = i < back ? sr[(size_t)i * C] : 0.f;
-    const int count = end - first;
-    auto z = [&](int idx) { return idx < back ? old[idx] : to_f32<TI>(x[(size_t)(first + idx - back) * ldx + c]); };
-    const int n_here = count < back ? count : back;
-    for (int m = 0; m < n_here; ++m) {
-        float acc = b0;
-        for (int j = 0; j < taps; ++j) acc = fmaf(wc[j], z(m + j), acc);
-        y[(size_t)(first + m) * ldy + c] = from_f32<TO>(finish(acc));
-    }
-    if (keep) {
-        float keep_v[CONV_MAX_TAPS];
-        for (int i = 0; i < back; ++i) keep_v[i] = z(count + i);
-        for (int i = 0; i < back; ++i) sr[(size_t)i * C] = keep_v[i];
-    }
+    y[(size_t)t * ldy + c] = from_f32<TO>(act == 1 ? acc / (1.0f + expf(-acc)) : acc);
 }
 
-// bfloat16 rows whose sizes let a thread take eight channels at a time (16-byte loads and stores).  The thread of an
-// entry's token further than taps - 2 into the entry reads rows of the step only; the others leave their eight
-// channels to the one-channel kernel's rule (see above), applied here channel by channel.
+// bfloat16 rows whose sizes let a thread take eight channels at a time (16-byte loads and stores); the same sums.
 #define CONV_VEC_TAPS 8
 __global__ __launch_bounds__(256)
 void causal_conv_vec_kernel(const bf16* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ bias,
-                            float* __restrict__ state, const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
-                            const int* __restrict__ seq_slots, bf16* __restrict__ y, int ldy, int C, int taps, int act, int keep) {
+                            const float* __restrict__ state, const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
+                            const int* __restrict__ seq_slots, bf16* __restrict__ y, int ldy, int C, int taps, int act) {
     const int t = blockIdx.x;
     const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
     if (c >= C) return;
     const int e = seq_of_token[t];
-    const int first = cu_seqlens[e], end = cu_seqlens[e + 1];
+    const int first = cu_seqlens[e];
     const int local = t - first, back = taps - 1;
-    auto finish = [&](float v) { return act == 1 ? v / (1.0f + expf(-v)) : v; };
-    if (local >= back) {
-        float acc[8];
+    const float* sr = state + (size_t)seq_slots[e] * back * C + c;
+    float acc[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = bias ? bias[c + i] : 0.f;
+    for (int i = 0; i < 8; ++i) acc[i] = bias ? bias[c + i] : 0.f;
 #pragma unroll
-        for (int j = 0; j < CONV_VEC_TAPS; ++j) {
-            if (j < taps) {
-                const bf16x8 xv = *(const bf16x8*)(x + (size_t)(t - back + j) * ldx + c);
+    for (int j = 0; j < CONV_VEC_TAPS; ++j) {
+        if (j < taps) {
+            const int r = local - back + j;
+            float u[8];
+            if (r >= 0) {
+                const bf16x8 xv = *(const bf16x8*)(x + (size_t)(first + r) * ldx + c);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) acc[i] = fmaf(w[(size_t)(c + i) * taps + j], (float)xv[i], acc[i]);
+                for (int i = 0; i < 8; ++i) u[i] = (float)xv[i];
+            } else {
+                const f32x4 s0 = *(const f32x4*)(sr + (size_t)(r + back) * C), s1 = *(const f32x4*)(sr + (size_t)(r + back) * C + 4);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { u[i] = s0[i]; u[4 + i] = s1[i]; }
             }
-        }
-        bf16x8 o;
+            const f32x4 w0 = *(const f32x4*)(w + (size_t)j * C + c), w1 = *(const f32x4*)(w + (size_t)j * C + c + 4);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] = (bf16)finish(acc[i]);
-        *(bf16x8*)(y + (size_t)t * ldy + c) = o;
-        return;
-    }
-    if (local != 0) return;
-    const int count = end - first;
-    const int n_here = count < back ? count : back;
-    for (int i = 0; i < 8; ++i) {
-        const int ci = c + i;
-        float* sr = state + (size_t)seq_slots[e] * back * C + ci;
-        float old[CONV_VEC_TAPS];
-        for (int k = 0; k < back; ++k) old[k] = sr[(size_t)k * C];
-        auto z = [&](int idx) { return idx < back ? old[idx] : (float)x[(size_t)(first + idx - back) * ldx + ci]; };
-        const float b0 = bias ? bias[ci] : 0.f;
-        for (int m = 0; m < n_here; ++m) {
-            float acc = b0;
-            for (int j = 0; j < taps; ++j) acc = fmaf(w[(size_t)ci * taps + j], z(m + j), acc);
-            y[(size_t)(first + m) * ldy + ci] = (bf16)finish(acc);
-        }
-        if (keep) {
-            float keep_v[CONV_VEC_TAPS];
-            for (int k = 0; k < back; ++k) keep_v[k] = z(count + k);
-            for (int k = 0; k < back; ++k) sr[(size_t)k * C] = keep_v[k];
+            for (int i = 0; i < 4; ++i) { acc[i] = fmaf(w0[i], u[i], acc[i]); acc[4 + i] = fmaf(w1[i], u[4 + i], acc[4 + i]); }
         }
     }
+    bf16x8 o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (bf16)(act == 1 ? acc[i] / (1.0f + expf(-acc[i])) : acc[i]);
+    *(bf16x8*)(y + (size_t)t * ldy + c) = o;
+}
+
+// The state after the step: the last taps - 1 inputs of (the old state, then the entry's rows).  A thread a (entry, channel).
+template <typename TI>
+__global__ __launch_bounds__(256)
+void causal_conv_keep_kernel(const TI* __restrict__ x, int ldx, float* __restrict__ state, const int* __restrict__ cu_seqlens,
+                             const int* __restrict__ seq_slots, int C, int taps) {
+    const int e = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int first = cu_seqlens[e], count = cu_seqlens[e + 1] - first, back = taps - 1;
+    float* sr = state + (size_t)seq_slots[e] * back * C + c;
+    float v[CONV_MAX_TAPS];
+#pragma unroll
+    for (int k = 0; k < CONV_MAX_TAPS; ++k) {
+        v[k] = 0.f;
+        if (k < back) {
+            const int idx = count + k;                     // among the old state's inputs (idx < back) or the entry's rows
+            v[k] = idx < back ? sr[(size_t)idx * C] : to_f32<TI>(x[(size_t)(first + idx - back) * ldx + c]);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < CONV_MAX_TAPS; ++k)
+        if (k < back) sr[(size_t)k * C] = v[k];
 }
 
 extern "C" int spite_causal_conv(const void* x, int ldx, int x_dtype, const float* w, const float* bias, float* state,
-                                 const int* seq_of_token, const int* cu_seqlens, const int* seq_slots, void* y, int ldy,
+                                 const int* seq_of_token, const int* cu_seqlens, const int* seq_slots, int n_seqs, void* y, int ldy,
                                  int y_dtype, int T, int C, int taps, int act, int keep, hipStream_t st) {
     SP_REQUIRE(T >= 0 && C > 0 && taps >= 1 && taps <= CONV_MAX_TAPS, "causal_conv: %d channels, %d taps (at most %d)", C, taps, CONV_MAX_TAPS);
     SP_REQUIRE(ldx >= C && ldy >= C && (act == 0 || act == 1), "causal_conv: rows shorter than the channels, or activation %d", act);
     SP_REQUIRE(taps == 1 || state, "causal_conv: the request's last inputs need a state");
+    SP_REQUIRE(n_seqs >= 0 && n_seqs <= T, "causal_conv: %d entries of %d tokens", n_seqs, T);
     if (T == 0) return 0;
-    if (x_dtype == SP_BF16 && y_dtype == SP_BF16 && C % 8 == 0 && ldx % 8 == 0 && ldy % 8 == 0 && taps <= CONV_VEC_TAPS
-        && ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 15) == 0) {
-        const dim3 vgrid(T, (C / 8 + 255) / 256);
-        causal_conv_vec_kernel<<<vgrid, 256, 0, st>>>((const bf16*)x, ldx, w, bias, state, seq_of_token, cu_seqlens, seq_slots,
-                                                      (bf16*)y, ldy, C, taps, act, keep);
-        SP_LAUNCH_CHECK("causal_conv");
-        return 0;
-    }
     const dim3 grid(T, (C + 255) / 256);
     SP_REQUIRE(grid.y <= 65535, "causal_conv: too many channels");
-#define SP_CC(TI, TO) causal_conv_kernel<TI, TO><<<grid, 256, 0, st>>>((const TI*)x, ldx, w, bias, state, seq_of_token, cu_seqlens, \
-        seq_slots, (TO*)y, ldy, C, taps, act, keep)
-    if (x_dtype == SP_F32 && y_dtype == SP_F32) SP_CC(float, float);
-    else if (x_dtype == SP_BF16 && y_dtype == SP_BF16) SP_CC(bf16, bf16);
-    else return sp_fail("causal_conv: dtypes %d -> %d", x_dtype, y_dtype);
-#undef SP_CC
+    if (x_dtype == SP_BF16 && y_dtype == SP_BF16 && C % 8 == 0 && ldx % 8 == 0 && ldy % 8 == 0 && taps <= CONV_VEC_TAPS
+        && ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 15) == 0 && ((uintptr_t)state & 15) == 0 && ((uintptr_t)w & 15) == 0) {
+        const dim3 vgrid(T, (C / 8 + 255) / 256);
+        causal_conv_vec_kernel<<<vgrid, 256, 0, st>>>((const bf16*)x, ldx, w, bias, state, seq_of_token, cu_seqlens, seq_slots,
+                                                      (bf16*)y, ldy, C, taps, act);
+    } else if (x_dtype == SP_F32 && y_dtype == SP_F32) {
+        causal_conv_kernel<float, float><<<grid, 256, 0, st>>>((const float*)x, ldx, w, bias, state, seq_of_token, cu_seqlens, seq_slots,
+                                                               (float*)y, ldy, C, taps, act);
+    } else if (x_dtype == SP_BF16 && y_dtype == SP_BF16) {
+        causal_conv_kernel<bf16, bf16><<<grid, 256, 0, st>>>((const bf16*)x, ldx, w, bias, state, seq_of_token, cu_seqlens, seq_slots,
+                                                             (bf16*)y, ldy, C, taps, act);
+    } else return sp_fail("causal_conv: dtypes %d -> %d", x_dtype, y_dtype);
     SP_LAUNCH_CHECK("causal_conv");
+    if (keep && taps > 1 && n_seqs > 0) {
+        const dim3 kgrid(n_seqs, (C + 255) / 256);
+        if (x_dtype == SP_F32) causal_conv_keep_kernel<float><<<kgrid, 256, 0, st>>>((const float*)x, ldx, state, cu_seqlens, seq_slots, C, taps);
+        else causal_conv_keep_kernel<bf16><<<kgrid, 256, 0, st>>>((const bf16*)x, ldx, state, cu_seqlens, seq_slots, C, taps);
+        SP_LAUNCH_CHECK("causal_conv (state)");
+    }
     return 0;
 }
 

@@ -79,7 +79,7 @@ def lib():
             "spite_add_tanh_norm_proj": [P, P, P, P, P, P, P, F, P, P, P, P, I, P, I, I, I, P, P, I, P],
             "spite_hash_rows": [P, P, P, P, P, P, P, I, ctypes.c_longlong, ctypes.c_longlong, ctypes.c_longlong, I, P],
             "spite_embed_sum": [P, P, P, P, I, P, I, I, I, I, F, P],
-            "spite_causal_conv": [P, I, I, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+            "spite_causal_conv": [P, I, I, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, P],
             "spite_shift_mix": [P, I, P, P, P, P, P, P, I, I, I, I, P],
             "spite_step_decay": [P, I, I, P, P, P, P, I, I, I, P],
             "spite_softcap_rows": [P, c_size_t, F, P],
@@ -1095,23 +1095,24 @@ CONV_ACTS = {None: 0, "silu": 1}
 
 
 def causal_conv(x, w, y, state, seq_of_token, cu_seqlens, seq_slots, bias=None, act=None, keep=True):
-    """y[t, c] = act(bias[c] + sum_j w[c, j] * x[t - taps + 1 + j, c]) within a request; the inputs before an entry's
+    """y[t, c] = act(bias[c] + sum_j w[j, c] * x[t - taps + 1 + j, c]) within a request; the inputs before an entry's
     first token come from state (fp32 [slots, taps-1, C]), which then holds the request's last taps - 1 inputs.  x and y:
-    [T, C] views of one dtype whose rows may lie apart; w fp32 [C, taps]."""
+    [T, C] views of one dtype whose rows may lie apart; w fp32 [taps, C], tap by tap (a checkpoint's [C, taps] transposed)."""
     T = y.shape[0]
-    C, taps = w.shape
+    taps, C = w.shape
     px, ldx = _rows_view(x, "x", C, T)
     py, ldy = _rows_view(y, "y", C, T)
     if x.dtype != y.dtype or act not in CONV_ACTS or (bias is not None and bias.numel() != C):
         raise KernelError("causal_conv: x and y of one dtype, activation silu or none, a bias per channel")
     if taps > 1 and (state is None or tuple(state.shape[1:]) != (taps - 1, C)):
         raise KernelError(f"causal_conv: state {None if state is None else tuple(state.shape)} for {taps} taps on {C} channels")
-    if seq_of_token.numel() < T:
-        raise KernelError("causal_conv: metadata too small")
+    if seq_of_token.numel() < T or cu_seqlens.numel() != seq_slots.numel() + 1:
+        raise KernelError("causal_conv: metadata too small, or not one more running count than entries")
     _check(lib().spite_causal_conv(px, ldx, dtype_code(x.dtype), _ptr(w, "w", torch.float32), _ptr(bias, "bias", torch.float32, True),
                                    _ptr(state, "state", torch.float32, True), _ptr(seq_of_token, "seq_of_token", torch.int32),
                                    _ptr(cu_seqlens, "cu_seqlens", torch.int32), _ptr(seq_slots, "seq_slots", torch.int32),
-                                   py, ldy, dtype_code(y.dtype), T, C, taps, CONV_ACTS[act], int(bool(keep)), _stream()), "causal_conv")
+                                   int(seq_slots.numel()), py, ldy, dtype_code(y.dtype), T, C, taps, CONV_ACTS[act], int(bool(keep)),
+                                   _stream()), "causal_conv")
 
 
 def shift_mix(x, mu, state, y, seq_of_token, cu_seqlens, seq_slots, keep=True):

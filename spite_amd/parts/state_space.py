@@ -57,7 +57,8 @@ class StateSpace(Mixer):
             w = torch.cat([w, torch.zeros((pad, w.shape[1]), dtype=w.dtype, device=w.device)], dim=0)
         self.rows_in = w.shape[0]
         self.w_in = Weight(w)
-        self.w_conv, self.b_conv = t["conv"].float().contiguous(), t["conv_bias"].float().contiguous()
+        # tap by tap, [taps, channels]: the kernel's loads of one tap are consecutive
+        self.w_conv, self.b_conv = t["conv"].float().t().contiguous(), t["conv_bias"].float().contiguous()
         self.dt_bias, self.a_log = t["dt_bias"].float().contiguous(), t["a_log"].float().contiguous()
         self.skip, self.w_norm = t["skip"].float().contiguous(), t["norm"].float().contiguous()
         self.wo = Weight(t["o_proj"])

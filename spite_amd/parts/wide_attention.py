@@ -164,7 +164,8 @@ class WideAttention(Mixer):
         if self.projection_norm or self.head_norm:
             self.w_qnorm, self.w_knorm = t["q_norm"].float().contiguous(), t["k_norm"].float().contiguous()
         if self.taps:
-            self.w_conv = torch.cat([t["q_conv"].float(), t["k_conv"].float()], dim=0).contiguous()
+            # tap by tap, [taps, channels]: the kernel's loads of one tap are consecutive
+            self.w_conv = torch.cat([t["q_conv"].float(), t["k_conv"].float()], dim=0).t().contiguous()
         if self.score_position is not None:
             self.slopes = self.score_position.score_slopes(self.HQ)
         if self.maps == 2:

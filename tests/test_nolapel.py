@@ -436,7 +436,7 @@ def test_convolution_kernel(dtype, taps, C, bias, act):
         wide[:, 3:3 + C] = torch.cat([u[i][fed[i]:fed[i] + lens[i]] for i in range(3)])
         wide = wide.cuda()
         y = torch.full((T, C), float("nan"), dtype=dt, device="cuda:0")
-        hipops.causal_conv(wide[:, 3:3 + C], w.cuda(), y, state, sot, cu, sl, bias=None if b is None else b.cuda(), act=act)
+        hipops.causal_conv(wide[:, 3:3 + C], w.t().contiguous().cuda(), y, state, sot, cu, sl, bias=None if b is None else b.cuda(), act=act)
         ref = torch.cat([want[i][fed[i]:fed[i] + lens[i]] for i in range(3)])
         tol = 1e-5 if dtype == "float32" else 2e-2
         assert float((y.cpu().double() - ref).abs().max()) <= tol * max(1.0, float(ref.abs().max()))
