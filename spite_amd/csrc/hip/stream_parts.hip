@@ -87,9 +87,10 @@ void add_tanh_norm_any_kernel(float* __restrict__ h, const float* __restrict__ d
 
 // The same with small fp32 products of the normed row formed on the way (router logits): a workgroup a row, the
 // normed row kept in LDS, proj_out[i][e] = proj[e] . normed row, a wave a product.  Rows of a multiple of four
-// elements that fit the LDS.
+// elements that fit the LDS.  Launched with 256 threads a row, or with 1,024 for a step of few rows (single tokens), where
+// a row's tanh evaluations are the time.
 template <typename TO>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(1024)
 void add_tanh_norm_proj_kernel(float* __restrict__ h, const float* __restrict__ d1, const float* __restrict__ d2,
                                const float* __restrict__ yn, const float* __restrict__ wn, const float* __restrict__ bn,
                                const float* __restrict__ alpha_n, float mult,
@@ -99,7 +100,7 @@ void add_tanh_norm_proj_kernel(float* __restrict__ h, const float* __restrict__ 
     extern __shared__ __attribute__((aligned(16))) float xs[];
     const size_t r = blockIdx.x;
     const float a = alpha[0], an = alpha_n ? alpha_n[0] : 0.f;
-    for (int c = threadIdx.x * 4; c < d; c += 1024) {
+    for (int c = threadIdx.x * 4; c < d; c += blockDim.x * 4) {
         f32x4 v = *(const f32x4*)(h + r * d + c);
         if (d1) v += *(const f32x4*)(d1 + r * d + c);
         if (d2) v += *(const f32x4*)(d2 + r * d + c);
@@ -126,7 +127,7 @@ void add_tanh_norm_proj_kernel(float* __restrict__ h, const float* __restrict__ 
     }
     __syncthreads();
     const int lane = threadIdx.x & 63;
-    for (int e = threadIdx.x >> 6; e < P; e += 4) {
+    for (int e = threadIdx.x >> 6; e < P; e += blockDim.x >> 6) {
         const float s = wave_dot_row(proj + (size_t)e * d, xs, d, true, lane);
         if (lane == 0) proj_out[r * P + e] = s;
     }
@@ -144,7 +145,8 @@ extern "C" int spite_add_tanh_norm_proj(float* h, const float* d1, const float* 
     SP_REQUIRE(al(h) && al(d1) && al(d2) && al(yn) && al(wn) && al(bn) && al(w) && al(b) && al(out32) && al(proj)
                && (out_dtype == SP_F32 ? al(out) : ((uintptr_t)out & 7) == 0), "add_tanh_norm: rows must start on 16 bytes");
     const size_t sh = (size_t)d * sizeof(float);
-#define SP_TNP(TO) add_tanh_norm_proj_kernel<TO><<<n_rows, 256, sh, st>>>(h, d1, d2, yn, wn, bn, alpha_n, mult, w, b, alpha, (TO*)out, out32, d, write_h, proj, proj_out, P)
+    const int threads = n_rows <= 256 && d >= 4096 ? 1024 : (n_rows <= 256 && d >= 2048 ? 512 : 256);
+#define SP_TNP(TO) add_tanh_norm_proj_kernel<TO><<<n_rows, threads, sh, st>>>(h, d1, d2, yn, wn, bn, alpha_n, mult, w, b, alpha, (TO*)out, out32, d, write_h, proj, proj_out, P)
     if (out_dtype == SP_F32) SP_TNP(float);
     else if (out_dtype == SP_BF16) SP_TNP(bf16);
     else return sp_fail("add_tanh_norm: unknown dtype %d", out_dtype);
