@@ -289,15 +289,15 @@ def nolapel_configs(sz, layers, window, vocab):
     groups = max(1, H // 8)
     ssm = ("mamba2", {"heads": H, "vdim": 128, "state": 128, "groups": groups, "conv": 4, "norm_groups": groups})
     attn = ("attention", {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "conv": 4,
-                          "mask": {"size": window}, "q_temp": {"coef": 0.3, "every": 1024}})
+                          "mask": {"size": window}, "q_temp": {"coef": 0.25, "every": 1024}})
     par = ("parallel", {"left": {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-                                 "rot": {"base": 1000000.0, "dims": 64}},
-                        "right": {"heads": H, "dim": 128}, "left_scale": 1.2, "right_scale": 0.9})
+                                 "rot": {"base": 500000.0, "dims": 64}},
+                        "right": {"heads": H, "dim": 128}, "left_scale": 1.1, "right_scale": 0.8})
     mixers = [ssm, attn, par, ssm]
     mlp = {"kind": "moe", "router": {"experts": sz["experts"], "top": sz["top"]}, "expert": {"ff": sz["expert_ff"]},
            "shared": {"ff": sz["shared_ff"]}}
-    nolapel = {"architecture": "Nolapel", "vocab": vocab, "width": sz["width"], "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
-               "embedding": {"bigram": {"buckets": 65521, "mul_prev": 127, "mul_cur": 17}}, "torch_dtype": "bfloat16",
+    nolapel = {"architecture": "Nolapel", "vocab": vocab, "width": sz["width"], "norm": {"eps": 1e-6}, "logit_softcap": 25.0,
+               "embedding": {"bigram": {"buckets": 65521, "mul_prev": 8191, "mul_cur": 31}}, "torch_dtype": "bfloat16",
                "loop": {"start": 0, "stop": min(2, layers), "times": 1},
                "layers": [{"type": mixers[i % 4][0], "mixer": mixers[i % 4][1], "mlp": mlp} for i in range(layers)]}
     return {"nolapel": nolapel, "tebalorn": tebalorn_configs(sz, layers, window, vocab)["tebalorn"]}

@@ -119,7 +119,7 @@ def cmd_bench(args) -> int:
 
 
 def main(argv=None) -> int:
-    ap = argparse.ArgumentParser(prog="spite", description="inference engine for one MI355X (Llama 4, Ravenex, Pefedra)")
+    ap = argparse.ArgumentParser(prog="spite", description="inference engine for one MI355X (Llama 4, Ravenex, Pefedra, Tebalorn, Nolapel)")
     sub = ap.add_subparsers(dest="cmd", required=True)
     run = sub.add_parser("run", help="generate tokens from a single prompt and print the output")
     _add_engine_args(run)

@@ -247,7 +247,7 @@ extern "C" int spite_embed_sum(const int* ids, const void* table, const int* row
 // behind this one, then leaves the request's last taps - 1 inputs in the state: one thread reads and writes a channel's
 // state, so entries of any length are safe.  Sums run over j upwards from the bias, the same for every token wherever
 // a request is cut.
-#define CONV_MAX_TAPS 16
+#define CONV_MAX_TAPS 32
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256)
 void causal_conv_kernel(const TI* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ bias,

@@ -152,9 +152,16 @@ class Model:
                 if ctx.n_out == 0:
                     state["logits"] = torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.env.device)
                     continue
-                d1, d2 = P.two_increments(state["h"], state["pending"])
+                pend, extra = state["pending"], {}
+                if getattr(self.final_norm, "takes_gathered", False):
+                    # the last layer's normed increment joins the wanted rows inside the final norm's own pass
+                    mine = [p for p in pend if isinstance(p, P.NORMED_INCREMENTS) and self.final_norm.takes(p)]
+                    if mine:
+                        extra["normed"] = mine[-1].as_arg()
+                        pend = tuple(p for p in pend if p is not mine[-1])
+                d1, d2 = P.two_increments(state["h"], pend)
                 rows = ctx.ws.take((ctx.n_out, d), self.env.dtype)
-                self.final_norm.forward(state["h"], rows, d1=d1, d2=d2, rows=ctx.logit_rows, write_h=False)
+                self.final_norm.forward(state["h"], rows, d1=d1, d2=d2, rows=ctx.logit_rows, write_h=False, **extra)
                 state["logits"] = step_ws.take((ctx.n_out, self.spec.vocab_size), torch.float32)
                 self.head.forward(rows, state["logits"], ctx)
         return state

@@ -59,6 +59,8 @@ class RMSNorm(Norm):
 @register("norm", "tanh")
 class TanhNorm(Norm):
     graph_safe = True
+    #: ``forward`` adds a normed increment also where it gathers rows and leaves the stream as it is (the model's last norm)
+    takes_gathered = True
 
     def __init__(self, env, width: int):
         self.width = int(width)

@@ -378,7 +378,7 @@ def test_hashed_embedding_kernels():
     """Two steps over slots that lie apart: the first token of a request takes the last row, the first token of a
     later portion hashes with the request's last token of the step before."""
     from spite_amd.csrc import hipops
-    V, d, buckets, mp, mc = 30, 12, 11, 127, 17
+    V, d, buckets, mp, mc = 30, 12, 11, 1009, 23
     g = torch.Generator().manual_seed(1)
     table, pairs = torch.randn(V, d, generator=g), torch.randn(buckets + 1, d, generator=g)
     seqs = [H.random_tokens(V, n, 3 + n) for n in (7, 1, 9)]
@@ -587,8 +587,8 @@ def test_decay_forms_and_small_row_kernels():
     out = torch.empty(5, 12, device="cuda:0")
     hipops.bias_rows(a, c[0].contiguous(), out)
     assert torch.equal(out.cpu(), a.cpu() + c[0].cpu())
-    want = 1.2 * a.cpu().double() + 0.9 * c.cpu().double()
-    hipops.axpby_rows(a, c, a, 1.2, 0.9)
+    want = 1.3 * a.cpu().double() + 0.6 * c.cpu().double()
+    hipops.axpby_rows(a, c, a, 1.3, 0.6)
     assert float((a.cpu().double() - want).abs().max()) < 1e-6
     for act_in in (torch.randn(6, 16, generator=g) * 3.0,):
         w = torch.randn(8, 16, generator=g)
@@ -985,7 +985,7 @@ def random_config(seed, aligned=False):
             dims = int(pick(*[x for x in (2, 4, 8, 16, 32, dim) if x <= dim and x % 2 == 0]))
             mixer = _parallel(heads, kv, dim, vdim, float(pick(0.1, 0.25)), pick(None, (float(pick(100.0, 10000.0, 1e6)), dims)),
                               int(pick(1, 2, 4)), int(pick(16, 32, 64)) if aligned else int(pick(2, 5, 8, 12)),
-                              ls=float(pick(1.0, 1.2, 0.5)), rs=float(pick(1.0, 0.9)))
+                              ls=float(pick(1.0, 1.3, 0.5)), rs=float(pick(1.0, 0.8)))
         else:
             groups = int(pick(1, 2))
             h = groups * int(pick(1, 2, 3))
@@ -1001,7 +1001,7 @@ def random_config(seed, aligned=False):
         a = int(rng.randint(len(layers)))
         cfg["loop"] = {"start": a, "stop": int(a + 1 + rng.randint(len(layers) - a)), "times": int(pick(1, 2, 3))}
     if pick(True, False):
-        cfg["logit_softcap"] = float(pick(5.0, 30.0))
+        cfg["logit_softcap"] = float(pick(5.0, 40.0))
     return cfg
 
 
