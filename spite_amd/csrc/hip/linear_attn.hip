@@ -335,6 +335,8 @@ extern "C" int spite_linear_attn_scan(const void* q, const void* k, const void* 
 // `pre_gate`: the gate comes before the norm, y = rmsnorm(o * act(gate)) * w.  `skip` (rows `lds` apart, in y's type)
 // with `skip_w` fp32 [n / skip_group]: o[c] + skip_w[c / skip_group] * skip[c] stands for o[c] (a direct path from
 // the recurrence's input to its result, one weight a head).
+#define GGN_KEEP 8            // values a lane keeps: groups of up to 512 elements are read once
+// (the wide form reads its values twice: holding up to 24 of them a thread was measured slower, 40 against 30 us)
 struct ggn_extra { const void* skip; int lds; const float* skip_w; int skip_group; int pre_gate; };
 template <typename TO>
 __device__ __forceinline__ float ggn_value(const float* orow, const TO* gate, int ldg, size_t t, int c0, int c, int act, const ggn_extra& ex) {
@@ -359,9 +361,28 @@ void gated_group_norm_kernel(const float* __restrict__ o, const TO* __restrict__
     const int c0 = (int)(item % groups) * group;
     const float* orow = o + t * n + c0;
     float ss = 0.f;
-    for (int c = lane; c < group; c += 64) { const float x = ggn_value<TO>(orow, gate, ldg, t, c0, c, act, ex); ss = fmaf(x, x, ss); }
+    float kept[GGN_KEEP];                             // a lane's first values stay in registers between the two passes
+#pragma unroll
+    for (int k = 0; k < GGN_KEEP; ++k) {
+        const int c = lane + k * 64;
+        kept[k] = c < group ? ggn_value<TO>(orow, gate, ldg, t, c0, c, act, ex) : 0.f;
+        ss = fmaf(kept[k], kept[k], ss);
+    }
+    for (int c = lane + GGN_KEEP * 64; c < group; c += 64) { const float x = ggn_value<TO>(orow, gate, ldg, t, c0, c, act, ex); ss = fmaf(x, x, ss); }
     const float sc = 1.0f / sqrtf(wave_sum(ss) / (float)group + eps);
-    for (int c = lane; c < group; c += 64) {
+#pragma unroll
+    for (int k = 0; k < GGN_KEEP; ++k) {
+        const int c = lane + k * 64;
+        if (c >= group) continue;
+        float x = kept[k] * sc * w[(c0 + c) % n_w];
+        if (act && !ex.pre_gate) {
+            const float g = to_f32<TO>(gate[t * ldg + c0 + c]);
+            const float sg = 1.0f / (1.0f + expf(-g));
+            x *= act == 1 ? g * sg : sg;
+        }
+        y[t * n + c0 + c] = from_f32<TO>(x);
+    }
+    for (int c = lane + GGN_KEEP * 64; c < group; c += 64) {
         float x = ggn_value<TO>(orow, gate, ldg, t, c0, c, act, ex) * sc * w[(c0 + c) % n_w];
         if (act && !ex.pre_gate) {
             const float g = to_f32<TO>(gate[t * ldg + c0 + c]);

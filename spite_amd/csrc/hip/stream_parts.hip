@@ -310,6 +310,93 @@ void causal_conv_vec_kernel(const bf16* __restrict__ x, int ldx, const float* __
     *(bf16x8*)(y + (size_t)t * ldy + c) = o;
 }
 
+// The same for steps of many tokens: a thread takes eight channels of CONV_TILE consecutive tokens, so a row is read once
+// for all the taps that use it and the weights once a tile.  A tile whose tokens belong to one entry runs as straight code
+// over rows held in registers; a tile across an entry's border falls back to the token-by-token form.  The sums are the
+// same in the same order.
+#define CONV_TILE 8
+template <int TAPS>
+__global__ __launch_bounds__(256)
+void causal_conv_tile_kernel(const bf16* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ bias,
+                             const float* __restrict__ state, const int* __restrict__ seq_of_token, const int* __restrict__ cu_seqlens,
+                             const int* __restrict__ seq_slots, bf16* __restrict__ y, int ldy, int C, int act, int T) {
+    constexpr int back = TAPS - 1;
+    const int t0 = blockIdx.x * CONV_TILE;
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+    if (c >= C) return;
+    const int n_tok = T - t0 < CONV_TILE ? T - t0 : CONV_TILE;
+    float wv[TAPS][8], bv[8];
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) {
+        const f32x4 w0 = *(const f32x4*)(w + (size_t)j * C + c), w1 = *(const f32x4*)(w + (size_t)j * C + c + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { wv[j][i] = w0[i]; wv[j][4 + i] = w1[i]; }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) bv[i] = bias ? bias[c + i] : 0.f;
+    auto row = [&](int e, int first, int r, float* u) {            // the input's row r, counted from the entry's first
+        if (r >= 0) {
+            const bf16x8 xv = *(const bf16x8*)(x + (size_t)(first + r) * ldx + c);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) u[i] = (float)xv[i];
+        } else {
+            const float* sr = state + ((size_t)seq_slots[e] * back + (r + back)) * C + c;
+            const f32x4 s0 = *(const f32x4*)sr, s1 = *(const f32x4*)(sr + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { u[i] = s0[i]; u[4 + i] = s1[i]; }
+        }
+    };
+    auto store = [&](int t, const float* acc) {
+        bf16x8 o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (bf16)(act == 1 ? acc[i] / (1.0f + expf(-acc[i])) : acc[i]);
+        *(bf16x8*)(y + (size_t)t * ldy + c) = o;
+    };
+    const int e0 = seq_of_token[t0];
+    if (e0 == seq_of_token[t0 + n_tok - 1]) {
+        const int first = cu_seqlens[e0], local0 = t0 - first;
+        float in[CONV_TILE + back][8];
+#pragma unroll
+        for (int k = 0; k < CONV_TILE + back; ++k) {
+            if (k - back < n_tok) row(e0, first, local0 - back + k, in[k]);
+            else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) in[k][i] = 0.f;
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < CONV_TILE; ++m) {
+            if (m < n_tok) {
+                float acc[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[i] = bv[i];
+#pragma unroll
+                for (int j = 0; j < TAPS; ++j) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc[i] = fmaf(wv[j][i], in[m + j][i], acc[i]);
+                }
+                store(t0 + m, acc);
+            }
+        }
+        return;
+    }
+    for (int m = 0; m < n_tok; ++m) {
+        const int t = t0 + m, e = seq_of_token[t];
+        const int first = cu_seqlens[e], local = t - first;
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = bv[i];
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
+            float u[8];
+            row(e, first, local - back + j, u);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = fmaf(wv[j][i], u[i], acc[i]);
+        }
+        store(t, acc);
+    }
+}
+
 // The state after the step: the last taps - 1 inputs of (the old state, then the entry's rows).  A thread a (entry, channel).
 template <typename TI>
 __global__ __launch_bounds__(256)
@@ -347,6 +434,15 @@ extern "C" int spite_causal_conv(const void* x, int ldx, int x_dtype, const floa
     if (x_dtype == SP_BF16 && y_dtype == SP_BF16 && C % 8 == 0 && ldx % 8 == 0 && ldy % 8 == 0 && taps <= CONV_VEC_TAPS
         && ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 15) == 0 && ((uintptr_t)state & 15) == 0 && ((uintptr_t)w & 15) == 0) {
         const dim3 vgrid(T, (C / 8 + 255) / 256);
+        const dim3 tgrid((T + CONV_TILE - 1) / CONV_TILE, (C / 8 + 255) / 256);
+#define SP_CT(N) causal_conv_tile_kernel<N><<<tgrid, 256, 0, st>>>((const bf16*)x, ldx, w, bias, state, seq_of_token, cu_seqlens, \
+        seq_slots, (bf16*)y, ldy, C, act, T)
+        // many tokens a step (portions of prompts): tiles of tokens; few (single tokens): a workgroup a token
+        if (T >= 32 * n_seqs && T >= 256 && taps == 4) SP_CT(4);
+        else if (T >= 32 * n_seqs && T >= 256 && taps == 3) SP_CT(3);
+        else if (T >= 32 * n_seqs && T >= 256 && taps == 2) SP_CT(2);
+        else
+#undef SP_CT
         causal_conv_vec_kernel<<<vgrid, 256, 0, st>>>((const bf16*)x, ldx, w, bias, state, seq_of_token, cu_seqlens, seq_slots,
                                                       (bf16*)y, ldy, C, taps, act);
     } else if (x_dtype == SP_F32 && y_dtype == SP_F32) {

@@ -449,6 +449,43 @@ def test_convolution_kernel(dtype, taps, C, bias, act):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("taps", [2, 3, 4])
+def test_convolution_kernel_in_tiles(taps):
+    """Steps of many tokens run in tiles of tokens: the same bits as the same requests in small portions (a workgroup a
+    token), tiles that cross an entry's border and a last tile that is not full included."""
+    from spite_amd.csrc import hipops
+    g = torch.Generator().manual_seed(taps)
+    C, lens = 40, [301, 5, 263]
+    u = [torch.randn(n, C, generator=g).to(torch.bfloat16) for n in lens]
+    w, b = torch.randn(C, taps, generator=g), torch.randn(C, generator=g)
+    wt = w.t().contiguous().cuda()
+    want = torch.cat([plain.silu(plain.causal_conv(x.double(), w.double(), b.double())) for x in u])
+    slots = [2, 0, 1]
+
+    def run(portion):
+        state = torch.zeros(3, taps - 1, C).cuda()
+        outs = [[] for _ in lens]
+        at = 0
+        while at < max(lens):
+            cut = [max(0, min(portion, n - at)) for n in lens]
+            live = [i for i, n in enumerate(cut) if n]
+            cu, sot, sl = _meta([cut[i] for i in live], [slots[i] for i in live])
+            rows = torch.cat([u[i][at:at + cut[i]] for i in live]).cuda()
+            y = torch.empty_like(rows)
+            hipops.causal_conv(rows, wt, y, state, sot, cu, sl, bias=b.cuda(), act="silu")
+            o = 0
+            for i in live:
+                outs[i].append(y[o:o + cut[i]].cpu())
+                o += cut[i]
+            at += portion
+        return torch.cat([torch.cat(x) for x in outs]), state.cpu()
+    whole, s1 = run(10 ** 6)
+    small, s2 = run(37)
+    assert torch.equal(whole, small) and torch.equal(s1, s2)
+    assert float((whole.double() - want).abs().max()) <= 2e-2 * max(1.0, float(want.abs().max()))
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_blend_with_the_row_before_kernel(dtype):
     from spite_amd.csrc import hipops
