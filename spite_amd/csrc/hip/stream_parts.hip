@@ -1,6 +1,6 @@
 // Parts around the residual stream that are no RMS norm and no attention:
 //
-//   add_tanh_norm:   residual additions + the "dynamic tanh" norm  y = tanh(alpha x) * w + b  (no mean, no variance),
+//   add_tanh_norm:   residual additions + the "dynamic tanh" norm  y = tanh(alpha x) * w + b  (each element on its own, no statistic of the row),
 //                    with one increment that passes such a norm of its own on its way into the stream
 //   hash_rows / embed_sum:  a second embedding whose row is a hash of (previous token, token); the previous token
 //                    of a request is kept in a state row

@@ -1,8 +1,8 @@
 """RMSNorm (crates/spite-models/src/dense.rs:175-181): y = x * 1/sqrt(mean(x^2) + eps) * w,
 sum and scale in fp32, fused with the residual additions that precede it.
 
-``tanh`` ("dynamic tanh"): y = tanh(alpha * x) * w + b with a learned scalar alpha: no mean, no variance, every
-element on its own; fp32, fused with the residual additions in the same way."""
+``tanh`` ("dynamic tanh"): y = tanh(alpha * x) * w + b with a learned scalar alpha: a squashing of every
+element on its own, without any statistic of the row; fp32, fused with the residual additions in the same way."""
 from __future__ import annotations
 
 import torch

@@ -26,7 +26,7 @@ def softplus(z):
 
 
 def dyt(x, W, name):
-    """Dynamic tanh: tanh(alpha x) * w + b; no mean, no variance."""
+    """The tanh norm: tanh(alpha x) * w + b, element by element."""
     return torch.tanh(W[name + ".alpha"] * x) * W[name] + W[name + ".b"]
 
 
