@@ -294,8 +294,7 @@ class ReentryBlock(Block):
     graph_safe = True
 
     def __init__(self, env, spec):
-        from .base import ParamSpec, PartSpec
-        from .norm import TanhNorm  # noqa: F401  (the increments' kinds are registered)
+        from .base import PartSpec
         self.env = env
         ex = spec.extra
         self.d, self.passes = int(ex["width"]), int(ex["passes"])
